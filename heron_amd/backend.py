@@ -1,0 +1,233 @@
+"""ctypes binding of ``librocm_heron.so`` (the C ABI declared in ``include/heron_rocm.h``).
+
+This is the only door to the kernels: there is no CPU fallback.  If the shared library is
+missing or a launch is attempted without a GPU, the calls raise ``HeronRocmError``.
+"""
+import ctypes
+import os
+import subprocess
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(_HERE, "csrc")
+LIB_PATH = os.path.join(CSRC, "librocm_heron.so")
+INCLUDE = os.path.join(os.path.dirname(_HERE), "include")
+
+HRN_DT_F16, HRN_DT_U8S8 = 0, 1
+HRN_OP_GEMM, HRN_OP_CONV2D = 0, 1
+HRN_OK = 0
+HRN_E_BADPARAM, HRN_E_BUILD, HRN_E_LOAD, HRN_E_LAUNCH, HRN_E_TIMEOUT, HRN_E_NODEVICE = -1, -2, -3, -4, -5, -6
+
+# flags every HIP translation unit of this package is compiled with
+HIPCC_FLAGS = ["--offload-arch=gfx950", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+class HeronRocmError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("hrn error %d: %s" % (code, msg))
+        self.code = code
+
+
+class DevInfo(ctypes.Structure):
+    _fields_ = [("arch", ctypes.c_char * 64), ("name", ctypes.c_char * 128),
+                ("cu_count", ctypes.c_int32), ("wave_size", ctypes.c_int32),
+                ("lds_bytes_per_wg", ctypes.c_int32), ("max_threads_per_wg", ctypes.c_int32),
+                ("clock_khz", ctypes.c_int32), ("mem_clock_khz", ctypes.c_int32),
+                ("mem_bus_bits", ctypes.c_int32), ("l2_bytes", ctypes.c_int32),
+                ("regs_per_simd_lane", ctypes.c_int32), ("simd_per_cu", ctypes.c_int32),
+                ("hbm_bytes", ctypes.c_uint64)]
+
+    def as_dict(self):
+        d = {}
+        for name, _ in self._fields_:
+            v = getattr(self, name)
+            d[name] = v.decode() if isinstance(v, bytes) else int(v)
+        return d
+
+
+class KernelDesc(ctypes.Structure):
+    _fields_ = [("dtype", ctypes.c_int32), ("op", ctypes.c_int32), ("bm", ctypes.c_int32), ("bn", ctypes.c_int32),
+                ("bkb", ctypes.c_int32), ("wm", ctypes.c_int32), ("wn", ctypes.c_int32), ("mfma", ctypes.c_int32),
+                ("stages", ctypes.c_int32), ("swizzle", ctypes.c_int32), ("epilogue", ctypes.c_int32),
+                ("waves_per_eu", ctypes.c_int32), ("reserved", ctypes.c_int32 * 4)]
+
+    KEYS = ("dtype", "op", "bm", "bn", "bkb", "wm", "wn", "mfma", "stages", "swizzle", "epilogue", "waves_per_eu")
+
+    def as_tuple(self):
+        return tuple(int(getattr(self, k)) for k in self.KEYS)
+
+    def __repr__(self):
+        return "KernelDesc(%s)" % ", ".join("%s=%d" % (k, getattr(self, k)) for k in self.KEYS)
+
+
+class KernelInfo(ctypes.Structure):
+    _fields_ = [("vgprs", ctypes.c_int32), ("agprs", ctypes.c_int32), ("sgprs", ctypes.c_int32),
+                ("lds_bytes", ctypes.c_int32), ("scratch_bytes", ctypes.c_int32), ("occupancy", ctypes.c_int32),
+                ("threads", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+    def as_dict(self):
+        return {n: int(getattr(self, n)) for n, _ in self._fields_ if n != "reserved"}
+
+
+class Problem(ctypes.Structure):
+    _fields_ = [("op", ctypes.c_int32), ("batch", ctypes.c_int32),
+                ("m", ctypes.c_int32), ("n", ctypes.c_int32), ("k", ctypes.c_int32),
+                ("lda", ctypes.c_int32), ("ldb", ctypes.c_int32), ("ldc", ctypes.c_int32),
+                ("stride_a", ctypes.c_int64), ("stride_b", ctypes.c_int64), ("stride_c", ctypes.c_int64),
+                ("cn", ctypes.c_int32), ("ch", ctypes.c_int32), ("cw", ctypes.c_int32), ("ci", ctypes.c_int32),
+                ("co", ctypes.c_int32), ("kh", ctypes.c_int32), ("kw", ctypes.c_int32),
+                ("cstride", ctypes.c_int32), ("cpad", ctypes.c_int32), ("cdil", ctypes.c_int32),
+                ("group_m", ctypes.c_int32), ("reserved", ctypes.c_int32 * 3)]
+
+
+def make_desc(dtype, op=HRN_OP_GEMM, bm=128, bn=128, bkb=128, wm=2, wn=2, mfma=32, stages=2, swizzle=1,
+              epilogue=0, waves_per_eu=0):
+    d = KernelDesc()
+    d.dtype, d.op, d.bm, d.bn, d.bkb, d.wm, d.wn = dtype, op, bm, bn, bkb, wm, wn
+    d.mfma, d.stages, d.swizzle, d.epilogue, d.waves_per_eu = mfma, stages, swizzle, epilogue, waves_per_eu
+    return d
+
+
+def build_library(force=True, verbose=False):
+    """Compile ``csrc/hrn_api.cpp`` into ``csrc/librocm_heron.so`` with hipcc (cross-compiles without a GPU)."""
+    if os.path.exists(LIB_PATH) and not force:
+        return LIB_PATH
+    hipcc = os.environ.get("HRN_HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, "-O2", "-fPIC", "-shared"] + HIPCC_FLAGS + [os.path.join(CSRC, "hrn_api.cpp"), "-o", LIB_PATH + ".tmp"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building librocm_heron.so failed:\n" + r.stderr[-4000:])
+    os.replace(LIB_PATH + ".tmp", LIB_PATH)
+    if verbose:
+        print("built", LIB_PATH)
+    global _lib
+    _lib = None
+    return LIB_PATH
+
+
+_lib = None
+_lock = threading.Lock()
+
+_vp, _i, _d = ctypes.c_void_p, ctypes.c_int, ctypes.c_double
+
+# every symbol include/heron_rocm.h declares: name -> (restype, argtypes)
+SYMBOLS = {
+    "hrn_device_info": (_i, [_i, ctypes.POINTER(DevInfo)]),
+    "hrn_check_desc": (_i, [ctypes.POINTER(KernelDesc)]),
+    "hrn_compile": (_i, [ctypes.POINTER(KernelDesc), _d, ctypes.c_char_p, ctypes.c_size_t]),
+    "hrn_build": (_i, [ctypes.POINTER(KernelDesc), _d, ctypes.POINTER(_vp)]),
+    "hrn_module_info": (_i, [_vp, ctypes.POINTER(KernelInfo)]),
+    "hrn_module_free": (None, [_vp]),
+    "hrn_lds_bytes": (_i, [ctypes.POINTER(KernelDesc)]),
+    "hrn_launch_gemm_f16": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
+    "hrn_launch_gemm_u8s8": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
+    "hrn_launch_bmm_f16": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
+    "hrn_launch_conv2d_nhwc_f16": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
+    "hrn_time": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _i, _d, ctypes.POINTER(_d), _vp]),
+    "hrn_problem_gemm": (None, [ctypes.POINTER(Problem), _i, _i, _i, _i]),
+    "hrn_problem_conv2d": (None, [ctypes.POINTER(Problem)] + [_i] * 10),
+    "hrn_last_error": (ctypes.c_char_p, []),
+    "hrn_version": (ctypes.c_char_p, []),
+}
+
+
+def lib():
+    """The loaded shared library; raises if it has not been built."""
+    global _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise HeronRocmError(HRN_E_LOAD, "%s is missing: run __graft_entry__.build() "
+                                     "(or heron_amd.backend.build_library())" % LIB_PATH)
+            L = ctypes.CDLL(LIB_PATH)
+            for name, (res, args) in SYMBOLS.items():
+                fn = getattr(L, name)
+                fn.restype = res
+                fn.argtypes = args
+            _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc != HRN_OK:
+        raise HeronRocmError(rc, lib().hrn_last_error().decode(errors="replace"))
+
+
+def device_info(device=0):
+    info = DevInfo()
+    _check(lib().hrn_device_info(device, ctypes.byref(info)))
+    return info.as_dict()
+
+
+def check_desc(desc):
+    """True when the descriptor satisfies the template's structural constraints."""
+    return lib().hrn_check_desc(ctypes.byref(desc)) == HRN_OK
+
+
+def lds_bytes(desc):
+    rc = lib().hrn_lds_bytes(ctypes.byref(desc))
+    if rc < 0:
+        _check(rc)
+    return rc
+
+
+def compile_desc(desc, timeout_s=0.0):
+    """hipcc the instance into the cache (no GPU needed); returns the code object path."""
+    buf = ctypes.create_string_buffer(1024)
+    _check(lib().hrn_compile(ctypes.byref(desc), float(timeout_s), buf, 1024))
+    return buf.value.decode()
+
+
+def gemm_problem(batch, m, n, k, group_m=8):
+    p = Problem()
+    lib().hrn_problem_gemm(ctypes.byref(p), batch, m, n, k)
+    p.group_m = group_m
+    return p
+
+
+def conv2d_problem(n, h, w, ci, co, kh, kw, stride, pad, dil, group_m=8):
+    p = Problem()
+    lib().hrn_problem_conv2d(ctypes.byref(p), n, h, w, ci, co, kh, kw, stride, pad, dil)
+    p.group_m = group_m
+    return p
+
+
+class Module:
+    """One loaded template instance (``hrn_module``)."""
+
+    def __init__(self, desc, timeout_s=0.0):
+        self.desc = desc
+        h = _vp()
+        _check(lib().hrn_build(ctypes.byref(desc), float(timeout_s), ctypes.byref(h)))
+        self._h = h
+        info = KernelInfo()
+        _check(lib().hrn_module_info(self._h, ctypes.byref(info)))
+        self.info = info.as_dict()
+
+    def _launcher(self, problem):
+        L = lib()
+        if self.desc.op == HRN_OP_CONV2D:
+            return L.hrn_launch_conv2d_nhwc_f16
+        if self.desc.dtype == HRN_DT_U8S8:
+            return L.hrn_launch_gemm_u8s8
+        return L.hrn_launch_bmm_f16 if problem.batch > 1 else L.hrn_launch_gemm_f16
+
+    def launch(self, problem, a_ptr, b_ptr, c_ptr, stream=0):
+        _check(self._launcher(problem)(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, stream))
+
+    def time(self, problem, a_ptr, b_ptr, c_ptr, number=3, repeat=4, min_repeat_ms=0.0, stream=0):
+        costs = (_d * repeat)()
+        _check(lib().hrn_time(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, number, repeat,
+                              float(min_repeat_ms), costs, stream))
+        return list(costs)
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().hrn_module_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,500 @@
+// C ABI of the gfx950 backend: template instantiation (hipcc -> code object cache), module
+// loading, launchers and event timing.  Declarations and the reference interfaces each entry
+// point stands in for are in include/heron_rocm.h.
+#include "../../include/heron_rocm.h"
+
+#include <hip/hip_runtime.h>
+
+#include <dlfcn.h>
+#include <fcntl.h>
+#include <signal.h>
+#include <sys/stat.h>
+#include <sys/types.h>
+#include <sys/wait.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <sstream>
+#include <string>
+#include <thread>
+#include <vector>
+
+#define HRN_KARGS_DEFINED
+struct HrnKArgs {  // must match mfma_gemm_template.hip
+    const void* A;
+    const void* B;
+    void* C;
+    int32_t M, N, K;
+    int32_t lda, ldb, ldc;
+    int64_t sA, sB, sC;
+    int32_t tiles_m, tiles_n, group_m, batch;
+    int32_t H, W, CI, HO, WO, KH, KW, cstride, cpad, cdil;
+    int32_t pad0, pad1;
+};
+
+struct hrn_module {
+    hrn_kernel_desc desc;
+    hrn_kernel_info info;
+    hipModule_t mod;
+    hipFunction_t fn;
+    std::string path;
+};
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[2048];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                         \
+    do {                                                                                      \
+        hipError_t e_ = (expr);                                                               \
+        if (e_ != hipSuccess) return fail(HRN_E_LAUNCH, "%s: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+std::string lib_dir() {
+    Dl_info di;
+    if (dladdr((void*)&hrn_last_error, &di) && di.dli_fname) {
+        std::string p = di.dli_fname;
+        size_t s = p.rfind('/');
+        return s == std::string::npos ? "." : p.substr(0, s);
+    }
+    return ".";
+}
+
+std::string env_or(const char* name, const std::string& dflt) {
+    const char* v = getenv(name);
+    return (v && *v) ? std::string(v) : dflt;
+}
+
+std::string kernel_source() { return env_or("HRN_KERNEL_DIR", lib_dir()) + "/mfma_gemm_template.hip"; }
+std::string cache_dir() { return env_or("HRN_CACHE_DIR", lib_dir() + "/cache"); }
+
+bool file_exists(const std::string& p) {
+    struct stat st;
+    return stat(p.c_str(), &st) == 0 && st.st_size > 0;
+}
+
+uint64_t fnv1a_file(const std::string& p) {
+    std::ifstream f(p, std::ios::binary);
+    uint64_t h = 1469598103934665603ull;
+    char buf[4096];
+    while (f) {
+        f.read(buf, sizeof buf);
+        for (std::streamsize i = 0; i < f.gcount(); ++i) { h ^= (unsigned char)buf[i]; h *= 1099511628211ull; }
+    }
+    return h;
+}
+
+struct Derived {
+    int es, nw, cpr, rpi, a_lpw, b_lpw, lpt, ksb, ks, tm, tn, stage_bytes, lds;
+};
+
+// Structural constraints of the template; the same conditions are static_asserts in the kernel.
+int derive(const hrn_kernel_desc* d, Derived* o) {
+    if (!d) return fail(HRN_E_BADPARAM, "null descriptor");
+    if (d->dtype != HRN_DT_F16 && d->dtype != HRN_DT_U8S8) return fail(HRN_E_BADPARAM, "dtype %d", d->dtype);
+    if (d->op != HRN_OP_GEMM && d->op != HRN_OP_CONV2D) return fail(HRN_E_BADPARAM, "op %d", d->op);
+    if (d->op == HRN_OP_CONV2D && d->dtype != HRN_DT_F16) return fail(HRN_E_BADPARAM, "conv2d is fp16 only");
+    if (d->bkb != 64 && d->bkb != 128 && d->bkb != 256) return fail(HRN_E_BADPARAM, "bkb %d not in {64,128,256}", d->bkb);
+    if (d->mfma != 32 && d->mfma != 16) return fail(HRN_E_BADPARAM, "mfma %d not in {16,32}", d->mfma);
+    if (d->wm < 1 || d->wn < 1 || d->wm * d->wn > 16) return fail(HRN_E_BADPARAM, "wave grid %dx%d", d->wm, d->wn);
+    if (d->bm < 16 || d->bn < 16 || d->bm > 512 || d->bn > 512) return fail(HRN_E_BADPARAM, "tile %dx%d", d->bm, d->bn);
+    if (d->stages < 2 || d->stages > 4) return fail(HRN_E_BADPARAM, "stages %d not in 2..4", d->stages);
+    if (d->swizzle < 0 || d->swizzle > 3) return fail(HRN_E_BADPARAM, "swizzle %d", d->swizzle);
+    if (d->epilogue < 0 || d->epilogue > 1) return fail(HRN_E_BADPARAM, "epilogue %d", d->epilogue);
+    if (d->waves_per_eu < 0 || d->waves_per_eu > 8) return fail(HRN_E_BADPARAM, "waves_per_eu %d", d->waves_per_eu);
+    Derived r;
+    r.es = d->dtype == HRN_DT_F16 ? 2 : 1;
+    r.nw = d->wm * d->wn;
+    r.cpr = d->bkb / 16;
+    r.rpi = 64 / r.cpr;
+    if (d->bm % r.rpi || d->bn % r.rpi || (d->bm / r.rpi) % r.nw || (d->bn / r.rpi) % r.nw)
+        return fail(HRN_E_BADPARAM, "tile rows must split evenly into 1 KiB wave loads (bm %d bn %d, %d rows/load, %d waves)",
+                    d->bm, d->bn, r.rpi, r.nw);
+    r.a_lpw = d->bm / r.rpi / r.nw;
+    r.b_lpw = d->bn / r.rpi / r.nw;
+    r.lpt = r.a_lpw + r.b_lpw;
+    r.ksb = d->mfma == 32 ? 32 : 64;
+    r.ks = d->bkb / r.ksb;
+    if (r.ks < 2 || r.ks % 2) return fail(HRN_E_BADPARAM, "bkb %d gives %d k-steps for mfma %d (need even >= 2)", d->bkb, r.ks, d->mfma);
+    if (d->bm % (d->wm * d->mfma) || d->bn % (d->wn * d->mfma))
+        return fail(HRN_E_BADPARAM, "tile %dx%d not divisible by wave grid %dx%d x mfma %d", d->bm, d->bn, d->wm, d->wn, d->mfma);
+    r.tm = d->bm / d->wm / d->mfma;
+    r.tn = d->bn / d->wn / d->mfma;
+    r.stage_bytes = (d->bm + d->bn) * d->bkb;
+    r.lds = d->stages * r.stage_bytes;
+    if (r.lds > 163840) return fail(HRN_E_BADPARAM, "LDS %d > 163840", r.lds);
+    if (d->swizzle && (r.cpr << (d->swizzle - 1)) > d->mfma)
+        return fail(HRN_E_BADPARAM, "swizzle %d period %d exceeds mfma %d", d->swizzle, r.cpr << (d->swizzle - 1), d->mfma);
+    if (d->op == HRN_OP_CONV2D && d->swizzle && (r.nw * r.rpi) % (r.cpr << (d->swizzle - 1)))
+        return fail(HRN_E_BADPARAM, "conv: swizzle period must divide rows per load round");
+    if ((d->stages - 1) * r.lpt > 63) return fail(HRN_E_BADPARAM, "too many loads in flight (%d)", (d->stages - 1) * r.lpt);
+    const int acc = r.tm * r.tn * (d->mfma == 32 ? 16 : 4);
+    if (acc > 256) return fail(HRN_E_BADPARAM, "accumulators %d > 256 registers per lane", acc);
+    if (d->dtype == HRN_DT_U8S8 && d->bn * 4 > r.lds) return fail(HRN_E_BADPARAM, "LDS too small for the column sums");
+    if (o) *o = r;
+    return HRN_OK;
+}
+
+std::string desc_key(const hrn_kernel_desc* d, uint64_t srch) {
+    char b[256];
+    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_%08x", d->dtype, d->op, d->bm, d->bn,
+             d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu,
+             (unsigned)(srch ^ (srch >> 32)));
+    return b;
+}
+
+int parse_remark(const std::string& log, const char* tag) {
+    size_t p = log.find(tag);
+    if (p == std::string::npos) return -1;
+    return atoi(log.c_str() + p + strlen(tag));
+}
+
+int run_hipcc(const std::vector<std::string>& args, const std::string& log_path, double timeout_s) {
+    pid_t pid = fork();
+    if (pid < 0) return fail(HRN_E_BUILD, "fork failed");
+    if (pid == 0) {
+        setpgid(0, 0);
+        int fd = open(log_path.c_str(), O_WRONLY | O_CREAT | O_TRUNC, 0644);
+        if (fd >= 0) { dup2(fd, 1); dup2(fd, 2); close(fd); }
+        std::vector<char*> argv;
+        for (auto& a : args) argv.push_back(const_cast<char*>(a.c_str()));
+        argv.push_back(nullptr);
+        execvp(argv[0], argv.data());
+        _exit(127);
+    }
+    auto t0 = std::chrono::steady_clock::now();
+    int status = 0;
+    for (;;) {
+        pid_t r = waitpid(pid, &status, WNOHANG);
+        if (r == pid) break;
+        if (r < 0) return fail(HRN_E_BUILD, "waitpid failed");
+        double el = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        if (timeout_s > 0 && el > timeout_s) {
+            kill(-pid, SIGKILL);
+            kill(pid, SIGKILL);
+            waitpid(pid, &status, 0);
+            return fail(HRN_E_TIMEOUT, "hipcc exceeded %.1f s", timeout_s);
+        }
+        std::this_thread::sleep_for(std::chrono::milliseconds(20));
+    }
+    if (!WIFEXITED(status) || WEXITSTATUS(status) != 0) {
+        std::ifstream f(log_path);
+        std::stringstream ss;
+        ss << f.rdbuf();
+        std::string s = ss.str();
+        if (s.size() > 1500) s = s.substr(0, 1500);
+        return fail(HRN_E_BUILD, "hipcc failed (status %d): %s", status, s.c_str());
+    }
+    return HRN_OK;
+}
+
+int compile_desc(const hrn_kernel_desc* d, double timeout_s, std::string* out_path) {
+    Derived dv;
+    int rc = derive(d, &dv);
+    if (rc) return rc;
+    const std::string src = kernel_source();
+    if (!file_exists(src)) return fail(HRN_E_BUILD, "kernel template not found: %s", src.c_str());
+    const std::string dir = cache_dir();
+    mkdir(dir.c_str(), 0755);
+    const std::string key = desc_key(d, fnv1a_file(src));
+    const std::string co = dir + "/" + key + ".hsaco";
+    const std::string info = dir + "/" + key + ".info";
+    *out_path = co;
+    if (file_exists(co) && file_exists(info)) return HRN_OK;
+
+    char tmp[64];
+    snprintf(tmp, sizeof tmp, ".tmp%d_%lx", (int)getpid(), (unsigned long)pthread_self());
+    const std::string co_tmp = co + tmp, log = dir + "/" + key + tmp + ".log";
+    std::vector<std::string> args = {env_or("HRN_HIPCC", "/opt/rocm/bin/hipcc"),
+                                     "--offload-arch=gfx950", "-O3", "--genco", "-std=c++17",
+                                     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                                     "-Rpass-analysis=kernel-resource-usage"};
+    auto def = [&](const char* n, int v) { args.push_back(std::string("-D") + n + "=" + std::to_string(v)); };
+    def("HRN_DTYPE", d->dtype); def("HRN_OP", d->op); def("HRN_BM", d->bm); def("HRN_BN", d->bn);
+    def("HRN_BKB", d->bkb); def("HRN_WM", d->wm); def("HRN_WN", d->wn); def("HRN_MFMA", d->mfma);
+    def("HRN_STAGES", d->stages); def("HRN_SWZ", d->swizzle); def("HRN_EPI", d->epilogue);
+    def("HRN_WPE", d->waves_per_eu);
+    args.push_back(src);
+    args.push_back("-o");
+    args.push_back(co_tmp);
+    rc = run_hipcc(args, log, timeout_s);
+    if (rc) { unlink(co_tmp.c_str()); unlink(log.c_str()); return rc; }
+
+    std::ifstream lf(log);
+    std::stringstream ss;
+    ss << lf.rdbuf();
+    const std::string ls = ss.str();
+    const std::string info_tmp = info + tmp;
+    {
+        std::ofstream o(info_tmp);
+        o << "vgprs " << parse_remark(ls, " VGPRs: ") << "\n"
+          << "agprs " << parse_remark(ls, "AGPRs: ") << "\n"
+          << "sgprs " << parse_remark(ls, "TotalSGPRs: ") << "\n"
+          << "scratch " << parse_remark(ls, "ScratchSize [bytes/lane]: ") << "\n"
+          << "occupancy " << parse_remark(ls, "Occupancy [waves/SIMD]: ") << "\n"
+          << "lds " << parse_remark(ls, "LDS Size [bytes/block]: ") << "\n";
+    }
+    unlink(log.c_str());
+    if (rename(co_tmp.c_str(), co.c_str()) != 0) return fail(HRN_E_BUILD, "rename %s failed", co.c_str());
+    rename(info_tmp.c_str(), info.c_str());
+    return HRN_OK;
+}
+
+void read_info(const std::string& path, hrn_kernel_info* o) {
+    std::ifstream f(path);
+    std::string k;
+    int v;
+    while (f >> k >> v) {
+        if (k == "vgprs") o->vgprs = v;
+        else if (k == "agprs") o->agprs = v;
+        else if (k == "sgprs") o->sgprs = v;
+        else if (k == "scratch") o->scratch_bytes = v;
+        else if (k == "occupancy") o->occupancy = v;
+        else if (k == "lds") o->lds_bytes = v;
+    }
+}
+
+int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, HrnKArgs* k,
+              unsigned* grid) {
+    if (!mod || !p || !A || !B || !C) return fail(HRN_E_BADPARAM, "null argument");
+    const hrn_kernel_desc& d = mod->desc;
+    if (p->op != d.op) return fail(HRN_E_BADPARAM, "problem op %d does not match module op %d", p->op, d.op);
+    const int es = d.dtype == HRN_DT_F16 ? 2 : 1;
+    memset(k, 0, sizeof *k);
+    k->A = A; k->B = B; k->C = C;
+    if (p->m <= 0 || p->n <= 0 || p->k <= 0 || p->batch <= 0) return fail(HRN_E_BADPARAM, "empty problem");
+    if ((int64_t)p->k * es % 16) return fail(HRN_E_BADPARAM, "K*%d must be a multiple of 16 bytes", es);
+    if (p->n % 4) return fail(HRN_E_BADPARAM, "N must be a multiple of 4");
+    k->M = p->m; k->N = p->n; k->K = p->k;
+    k->lda = p->lda; k->ldb = p->ldb; k->ldc = p->ldc;
+    k->sA = p->stride_a; k->sB = p->stride_b; k->sC = p->stride_c;
+    k->batch = p->batch;
+    if ((int64_t)p->ldb * es % 16 || p->ldb < p->k) return fail(HRN_E_BADPARAM, "ldb %d", p->ldb);
+    if (p->ldc % 4 || p->ldc < p->n) return fail(HRN_E_BADPARAM, "ldc %d", p->ldc);
+    if ((int64_t)p->n * p->ldb * es >= (1ll << 31)) return fail(HRN_E_BADPARAM, "B operand exceeds 2 GiB per batch entry");
+    if (d.op == HRN_OP_GEMM) {
+        if ((int64_t)p->lda * es % 16 || p->lda < p->k) return fail(HRN_E_BADPARAM, "lda %d", p->lda);
+        if ((int64_t)p->m * p->lda * es >= (1ll << 31)) return fail(HRN_E_BADPARAM, "A operand exceeds 2 GiB per batch entry");
+    } else {
+        if (p->batch != 1) return fail(HRN_E_BADPARAM, "conv batch is the image count");
+        if (p->cstride < 1 || p->cdil < 1 || p->cpad < 0) return fail(HRN_E_BADPARAM, "conv stride/pad/dilation");
+        const int ho = (p->ch - ((p->kh - 1) * p->cdil + 1) + 2 * p->cpad) / p->cstride + 1;
+        const int wo = (p->cw - ((p->kw - 1) * p->cdil + 1) + 2 * p->cpad) / p->cstride + 1;
+        if (ho <= 0 || wo <= 0) return fail(HRN_E_BADPARAM, "conv output is empty");
+        if (p->m != p->cn * ho * wo || p->n != p->co || p->k != p->kh * p->kw * p->ci)
+            return fail(HRN_E_BADPARAM, "conv GEMM view (m,n,k)=(%d,%d,%d) inconsistent with the image shape", p->m, p->n, p->k);
+        if ((p->ci * es) % 16) return fail(HRN_E_BADPARAM, "CI*%d must be a multiple of 16 bytes", es);
+        if ((int64_t)p->cn * p->ch * p->cw * p->ci * es >= (1ll << 31)) return fail(HRN_E_BADPARAM, "input exceeds 2 GiB");
+        k->H = p->ch; k->W = p->cw; k->CI = p->ci; k->HO = ho; k->WO = wo; k->KH = p->kh; k->KW = p->kw;
+        k->cstride = p->cstride; k->cpad = p->cpad; k->cdil = p->cdil;
+    }
+    k->tiles_m = (p->m + d.bm - 1) / d.bm;
+    k->tiles_n = (p->n + d.bn - 1) / d.bn;
+    k->group_m = p->group_m > 0 ? p->group_m : 8;
+    const int64_t total = (int64_t)k->tiles_m * k->tiles_n * p->batch;
+    if (total <= 0 || total >= (1ll << 31)) return fail(HRN_E_BADPARAM, "grid size");
+    *grid = (unsigned)total;
+    return HRN_OK;
+}
+
+int launch(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream) {
+    HrnKArgs k;
+    unsigned grid;
+    int rc = fill_args(mod, p, A, B, C, &k, &grid);
+    if (rc) return rc;
+    size_t sz = sizeof k;
+    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &k, HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
+    HIP_TRY(hipModuleLaunchKernel(mod->fn, grid, 1, 1, (unsigned)mod->info.threads, 1, 1, 0, (hipStream_t)stream,
+                                  nullptr, extra));
+    return HRN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* hrn_last_error(void) { return g_err.c_str(); }
+const char* hrn_version(void) { return "heron-rocm 0.1 (gfx950)"; }
+
+int hrn_device_info(int device, hrn_devinfo* out) {
+    if (!out) return fail(HRN_E_BADPARAM, "null out");
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return fail(HRN_E_NODEVICE, "no HIP device");
+    if (device < 0 || device >= n) return fail(HRN_E_BADPARAM, "device %d of %d", device, n);
+    hipDeviceProp_t pr;
+    HIP_TRY(hipGetDeviceProperties(&pr, device));
+    memset(out, 0, sizeof *out);
+    snprintf(out->arch, sizeof out->arch, "%s", pr.gcnArchName);
+    snprintf(out->name, sizeof out->name, "%s", pr.name);
+    out->cu_count = pr.multiProcessorCount;
+    out->wave_size = pr.warpSize;
+    out->lds_bytes_per_wg = (int32_t)pr.sharedMemPerBlock;
+    out->max_threads_per_wg = pr.maxThreadsPerBlock;
+    out->clock_khz = pr.clockRate;
+    out->mem_clock_khz = pr.memoryClockRate;
+    out->mem_bus_bits = pr.memoryBusWidth;
+    out->l2_bytes = pr.l2CacheSize;
+    out->regs_per_simd_lane = 512;
+    out->simd_per_cu = 4;
+    out->hbm_bytes = pr.totalGlobalMem;
+    return HRN_OK;
+}
+
+int hrn_check_desc(const hrn_kernel_desc* desc) { return derive(desc, nullptr); }
+
+int hrn_lds_bytes(const hrn_kernel_desc* desc) {
+    Derived d;
+    int rc = derive(desc, &d);
+    return rc ? rc : d.lds;
+}
+
+int hrn_compile(const hrn_kernel_desc* desc, double timeout_s, char* path_out, size_t path_cap) {
+    std::string path;
+    int rc = compile_desc(desc, timeout_s, &path);
+    if (rc) return rc;
+    if (path_out && path_cap) snprintf(path_out, path_cap, "%s", path.c_str());
+    return HRN_OK;
+}
+
+int hrn_build(const hrn_kernel_desc* desc, double timeout_s, hrn_module** out) {
+    if (!out) return fail(HRN_E_BADPARAM, "null out");
+    *out = nullptr;
+    std::string path;
+    int rc = compile_desc(desc, timeout_s, &path);
+    if (rc) return rc;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return fail(HRN_E_NODEVICE, "no HIP device");
+    hrn_module* m = new hrn_module();
+    m->desc = *desc;
+    m->path = path;
+    memset(&m->info, 0, sizeof m->info);
+    read_info(path.substr(0, path.size() - 6) + ".info", &m->info);
+    m->info.threads = desc->wm * desc->wn * 64;
+    hipError_t e = hipModuleLoad(&m->mod, path.c_str());
+    if (e != hipSuccess) {
+        delete m;
+        return fail(HRN_E_LOAD, "hipModuleLoad(%s): %s", path.c_str(), hipGetErrorString(e));
+    }
+    e = hipModuleGetFunction(&m->fn, m->mod, "hrn_mfma_kernel");
+    if (e != hipSuccess) {
+        (void)hipModuleUnload(m->mod);
+        delete m;
+        return fail(HRN_E_LOAD, "hipModuleGetFunction: %s", hipGetErrorString(e));
+    }
+    *out = m;
+    return HRN_OK;
+}
+
+int hrn_module_info(const hrn_module* mod, hrn_kernel_info* out) {
+    if (!mod || !out) return fail(HRN_E_BADPARAM, "null argument");
+    *out = mod->info;
+    return HRN_OK;
+}
+
+void hrn_module_free(hrn_module* mod) {
+    if (!mod) return;
+    (void)hipModuleUnload(mod->mod);
+    delete mod;
+}
+
+int hrn_launch_gemm_f16(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream) {
+    if (mod && (mod->desc.dtype != HRN_DT_F16 || mod->desc.op != HRN_OP_GEMM)) return fail(HRN_E_BADPARAM, "module is not an fp16 GEMM");
+    if (p && p->batch != 1) return fail(HRN_E_BADPARAM, "gemm takes batch 1 (use hrn_launch_bmm_f16)");
+    return launch(mod, p, A, B, C, stream);
+}
+
+int hrn_launch_gemm_u8s8(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream) {
+    if (mod && (mod->desc.dtype != HRN_DT_U8S8 || mod->desc.op != HRN_OP_GEMM)) return fail(HRN_E_BADPARAM, "module is not a u8s8 GEMM");
+    return launch(mod, p, A, B, C, stream);
+}
+
+int hrn_launch_bmm_f16(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream) {
+    if (mod && (mod->desc.dtype != HRN_DT_F16 || mod->desc.op != HRN_OP_GEMM)) return fail(HRN_E_BADPARAM, "module is not an fp16 GEMM");
+    return launch(mod, p, A, B, C, stream);
+}
+
+int hrn_launch_conv2d_nhwc_f16(const hrn_module* mod, const hrn_problem* p, const void* In, const void* Filter, void* Out, void* stream) {
+    if (mod && (mod->desc.dtype != HRN_DT_F16 || mod->desc.op != HRN_OP_CONV2D)) return fail(HRN_E_BADPARAM, "module is not an fp16 conv2d");
+    return launch(mod, p, In, Filter, Out, stream);
+}
+
+int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, int number, int repeat,
+             double min_repeat_ms, double* costs_out, void* stream) {
+    if (!costs_out || number < 1 || repeat < 1) return fail(HRN_E_BADPARAM, "number/repeat/costs_out");
+    HrnKArgs k;
+    unsigned grid;
+    int rc = fill_args(mod, p, A, B, C, &k, &grid);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    auto cleanup = [&]() { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); };
+    rc = launch(mod, p, A, B, C, stream);  // warm-up, also surfaces launch errors
+    if (rc) { cleanup(); return rc; }
+    if (hipStreamSynchronize(st) != hipSuccess) { cleanup(); return fail(HRN_E_LAUNCH, "warm-up failed: %s", hipGetErrorString(hipGetLastError())); }
+    for (int r = 0; r < repeat; ++r) {
+        int num = number;
+        for (;;) {
+            (void)hipEventRecord(e0, st);
+            for (int i = 0; i < num; ++i) {
+                rc = launch(mod, p, A, B, C, stream);
+                if (rc) { cleanup(); return rc; }
+            }
+            (void)hipEventRecord(e1, st);
+            if (hipEventSynchronize(e1) != hipSuccess) { cleanup(); return fail(HRN_E_LAUNCH, "kernel failed: %s", hipGetErrorString(hipGetLastError())); }
+            float ms = 0;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            if (ms >= min_repeat_ms || num >= (1 << 20)) {
+                costs_out[r] = (double)ms * 1e-3 / num;
+                number = num;  // keep the grown count for the next repeats
+                break;
+            }
+            // grow like time_evaluator: aim past min_repeat_ms with some margin
+            const double per = std::max((double)ms / num, 1e-4);
+            num = std::max(num + 1, (int)std::min(1048576.0, min_repeat_ms * 1.2 / per + 1));
+        }
+    }
+    cleanup();
+    return HRN_OK;
+}
+
+void hrn_problem_gemm(hrn_problem* p, int batch, int m, int n, int k) {
+    memset(p, 0, sizeof *p);
+    p->op = HRN_OP_GEMM;
+    p->batch = batch; p->m = m; p->n = n; p->k = k;
+    p->lda = k; p->ldb = k; p->ldc = n;
+    p->stride_a = (int64_t)m * k; p->stride_b = (int64_t)n * k; p->stride_c = (int64_t)m * n;
+    p->group_m = 8;
+}
+
+void hrn_problem_conv2d(hrn_problem* p, int n, int h, int w, int ci, int co, int kh, int kw, int stride, int pad, int dil) {
+    memset(p, 0, sizeof *p);
+    p->op = HRN_OP_CONV2D;
+    p->batch = 1;
+    p->cn = n; p->ch = h; p->cw = w; p->ci = ci; p->co = co; p->kh = kh; p->kw = kw;
+    p->cstride = stride; p->cpad = pad; p->cdil = dil;
+    const int ho = (stride > 0) ? (h - ((kh - 1) * dil + 1) + 2 * pad) / stride + 1 : 0;
+    const int wo = (stride > 0) ? (w - ((kw - 1) * dil + 1) + 2 * pad) / stride + 1 : 0;
+    p->m = n * ho * wo; p->n = co; p->k = kh * kw * ci;
+    p->lda = ci; p->ldb = p->k; p->ldc = co;
+    p->group_m = 8;
+}
+
+}  // extern "C"

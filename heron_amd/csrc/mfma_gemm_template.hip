@@ -1,0 +1,397 @@
+// MFMA tile-GEMM kernel template for gfx950 (CDNA4, wave64).
+//
+// One source, instantiated by -D macros (one instance = one point of the tuner's search space):
+//   HRN_DTYPE   0: fp16 x fp16 -> fp32 accumulate -> fp16 store      (ops/cuda/dense.py:4-54)
+//               1: uint8 x int8 -> int32 accumulate -> int32 store   (ops/x86/dense.py:6-32)
+//   HRN_OP      0: GEMM / batch_matmul   C[b,i,j] = sum_k A[b,i,k] * B[b,j,k]
+//               1: conv2d NHWC x KRSC as implicit GEMM (M = n*ho*wo, N = co, K = kh*kw*ci)
+//   HRN_BM/BN   workgroup tile, HRN_BKB bytes of K per LDS row, HRN_WM x HRN_WN wave grid,
+//   HRN_MFMA    32 | 16 (MFMA tile edge), HRN_STAGES LDS stages, HRN_SWZ LDS chunk swizzle,
+//   HRN_EPI     0 register epilogue, 1 LDS-staged epilogue, HRN_WPE waves-per-SIMD hint.
+//
+// Data movement: both operands are K-contiguous, so a tile is a set of rows of HRN_BKB bytes.
+// Rows are cut into 16-byte chunks; every lane moves one chunk per load straight from HBM/L2
+// into LDS (buffer_load_dwordx4 ... lds), one wave instruction filling 1 KiB of consecutive LDS.
+// The chunk a lane fetches is XOR-swizzled so that the MFMA operand reads (ds_read_b128, one
+// 16-byte chunk per lane) spread over all LDS banks.  Out-of-range rows, conv halo taps and the
+// dummy tiles past the end of K are fetched with an out-of-range buffer offset, which the
+// buffer unit turns into zeros.
+//
+// Pipeline: HRN_STAGES tiles are in flight.  The barrier that publishes tile t+1 sits before the
+// last k-step of tile t, so operand fragments of the next tile are already being read while the
+// last MFMAs of the current tile run; fragments are double-buffered in registers.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <type_traits>
+
+#ifndef HRN_DTYPE
+#error "instantiate with -DHRN_DTYPE=... (see hrn_api.cpp)"
+#endif
+
+#ifndef HRN_KARGS_DEFINED
+#define HRN_KARGS_DEFINED
+struct HrnKArgs {
+    const void* A;
+    const void* B;
+    void* C;
+    int32_t M, N, K;            // K in elements
+    int32_t lda, ldb, ldc;      // elements
+    int64_t sA, sB, sC;         // batch strides, elements
+    int32_t tiles_m, tiles_n, group_m, batch;
+    // conv
+    int32_t H, W, CI, HO, WO, KH, KW, cstride, cpad, cdil;
+    int32_t pad0, pad1;
+};
+#endif
+
+namespace {
+
+constexpr int DT = HRN_DTYPE;
+constexpr int OP = HRN_OP;
+constexpr int BM = HRN_BM, BN = HRN_BN, BKB = HRN_BKB;
+constexpr int WM = HRN_WM, WN = HRN_WN, MT = HRN_MFMA, NS = HRN_STAGES, SWZ = HRN_SWZ;
+constexpr int EPI = HRN_EPI;
+constexpr int ES = (DT == 0) ? 2 : 1;       // input element bytes
+constexpr int OES = (DT == 0) ? 2 : 4;      // output element bytes
+constexpr int NW = WM * WN, NT = NW * 64;
+constexpr int CPR = BKB / 16;               // 16-byte chunks per tile row
+constexpr int RPI = 64 / CPR;               // tile rows one wave load instruction covers
+constexpr int A_LPW = (BM / RPI) / NW;      // load instructions per wave per tile
+constexpr int B_LPW = (BN / RPI) / NW;
+constexpr int LPT = A_LPW + B_LPW;
+constexpr int KSB = (MT == 32) ? 32 : 64;   // bytes of K one MFMA consumes
+constexpr int KS = BKB / KSB;               // MFMA k-steps per tile
+constexpr int CPS = KSB / 16;               // chunks per k-step (= 64 / MT)
+constexpr int WTM = BM / WM, WTN = BN / WN;
+constexpr int TM = WTM / MT, TN = WTN / MT;
+constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB, STAGE_BYTES = A_BYTES + B_BYTES;
+constexpr int ACC_N = (MT == 32) ? 16 : 4;
+constexpr uint32_t OOB = 0x80000000u;
+
+static_assert(BKB == 64 || BKB == 128 || BKB == 256, "BKB");
+static_assert(MT == 32 || MT == 16, "MFMA");
+static_assert(KS >= 2 && (KS % 2) == 0, "need an even number of k-steps per tile");
+static_assert((BM / RPI) % NW == 0 && (BN / RPI) % NW == 0 && A_LPW >= 1 && B_LPW >= 1, "loads per wave");
+static_assert(BM % (WM * MT) == 0 && BN % (WN * MT) == 0, "wave tile");
+static_assert(NS >= 2 && NS <= 4, "stages");
+static_assert(NS * STAGE_BYTES <= 163840, "LDS");
+static_assert(SWZ == 0 || (CPR << (SWZ - 1)) <= MT, "swizzle period must fit in one MFMA tile");
+static_assert((NS - 1) * LPT <= 63, "vmcnt range");
+static_assert(NT <= 1024, "threads");
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+template <int N> struct AccT;
+template <> struct AccT<16> { using F = v16f; using I = v16i; };
+template <> struct AccT<4> { using F = v4f; using I = v4i; };
+using acc_t = typename std::conditional<DT == 0, typename AccT<ACC_N>::F, typename AccT<ACC_N>::I>::type;
+
+__device__ __forceinline__ int swz_of_row(int row) {
+    if (SWZ == 0) return 0;
+    return (row >> (SWZ - 1)) & (CPR - 1);
+}
+
+// s_waitcnt encodings for gfx9: vmcnt[3:0]|[15:14], expcnt[6:4], lgkmcnt[11:8]
+template <int VM, int LGKM>
+__device__ __forceinline__ void wait_and_barrier() {
+    constexpr int vm = VM > 63 ? 63 : VM;
+    constexpr int imm = (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((LGKM & 15) << 8);
+    asm volatile("s_waitcnt %0\n\ts_barrier" ::"n"(imm) : "memory");
+}
+
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+// raw buffer (stride 0): an offset >= `bytes` reads as zero instead of touching memory
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+__device__ __forceinline__ void load_chunk_to_lds(rsrc_t rsrc, char* lds_wave_base, uint32_t voff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds_wave_base,
+                                             16, (int)voff, 0, 0, 0);
+}
+
+__device__ __forceinline__ v16f mfma(v4i x, v4i y, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, x), __builtin_bit_cast(v8h, y), c, 0, 0, 0);
+}
+__device__ __forceinline__ v4f mfma(v4i x, v4i y, v4f c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, x), __builtin_bit_cast(v8h, y), c, 0, 0, 0);
+}
+__device__ __forceinline__ v16i mfma(v4i x, v4i y, v16i c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(x, y, c, 0, 0, 0);
+}
+__device__ __forceinline__ v4i mfma(v4i x, v4i y, v4i c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(x, y, c, 0, 0, 0);
+}
+
+// Scheduling pattern of one k-step: NR groups of {1 LDS read, NV/NR buffer loads, NMM/NR MFMAs}.
+template <int R, int NR, int NMM, int NV>
+__device__ __forceinline__ void sched_pattern() {
+    if constexpr (R < NR) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        constexpr int v = (NV * (R + 1)) / NR - (NV * R) / NR;
+        if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);
+        constexpr int mm = (NMM * (R + 1)) / NR - (NMM * R) / NR;
+        if constexpr (mm > 0) __builtin_amdgcn_sched_group_barrier(0x008, mm, 0);
+        sched_pattern<R + 1, NR, NMM, NV>();
+    }
+}
+
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(NT)
+#if HRN_WPE > 0
+__attribute__((amdgpu_waves_per_eu(HRN_WPE, HRN_WPE)))
+#endif
+hrn_mfma_kernel(const HrnKArgs a) {
+    __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm_idx = wave / WN, wn_idx = wave % WN;
+
+    // ---- tile raster: spread over the 8 XCDs so that each XCD's L2 sees a compact block ----
+    const int tiles_mn = a.tiles_m * a.tiles_n;
+    const int total = tiles_mn * a.batch;
+    int pid = blockIdx.x;
+    if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+    const int bz = pid / tiles_mn;
+    const int t = pid - bz * tiles_mn;
+    const int group_sz = a.group_m * a.tiles_n;
+    const int gid = t / group_sz;
+    const int first_m = gid * a.group_m;
+    const int gsz = min(a.tiles_m - first_m, a.group_m);
+    const int tin = t - gid * group_sz;
+    const int tile_m = first_m + tin % gsz;
+    const int tile_n = tin / gsz;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const char* Ab = (const char*)a.A + (int64_t)bz * a.sA * ES;
+    const char* Bb = (const char*)a.B + (int64_t)bz * a.sB * ES;
+    const uint32_t Kb = (uint32_t)a.K * ES;           // bytes of K
+    const int KT = (Kb + BKB - 1) / BKB;
+
+    uint32_t a_bytes, b_bytes = (uint32_t)a.N * (uint32_t)a.ldb * ES;
+    if constexpr (OP == 0) a_bytes = (uint32_t)a.M * (uint32_t)a.lda * ES;
+    else a_bytes = (uint32_t)(a.M / (a.HO * a.WO)) * (uint32_t)(a.H * a.W * a.CI) * ES;
+    const rsrc_t rsrcA = make_rsrc(Ab, a_bytes);
+    const rsrc_t rsrcB = make_rsrc(Bb, b_bytes);
+
+    // ---- per-lane load bookkeeping ----
+    const int lrow = lane / CPR, lpos = lane % CPR;
+    uint32_t voffB[B_LPW];
+#pragma unroll
+    for (int i = 0; i < B_LPW; ++i) {
+        const int row = (i * NW + wave) * RPI + lrow;
+        const int chunk = lpos ^ swz_of_row(row);
+        const int n = n0 + row;
+        voffB[i] = (n < a.N) ? (uint32_t)n * (uint32_t)a.ldb * ES + chunk * 16 : OOB;
+    }
+    // GEMM: byte offset of the lane's chunk in k-tile 0.  Conv: pixel bookkeeping.
+    uint32_t voffA[A_LPW];
+    int iy0[OP == 1 ? A_LPW : 1], ix0[OP == 1 ? A_LPW : 1];
+    int cc = 0, cs = 0, cr = 0;  // conv: channel / kw / kh position of the lane's chunk
+    if constexpr (OP == 0) {
+#pragma unroll
+        for (int i = 0; i < A_LPW; ++i) {
+            const int row = (i * NW + wave) * RPI + lrow;
+            const int chunk = lpos ^ swz_of_row(row);
+            const int m = m0 + row;
+            voffA[i] = (m < a.M) ? (uint32_t)m * (uint32_t)a.lda * ES + chunk * 16 : OOB;
+        }
+    } else {
+        static_assert(OP == 0 || SWZ == 0 || ((NW * RPI) % (CPR << (SWZ > 0 ? SWZ - 1 : 0))) == 0,
+                      "conv: the lane's chunk column must not depend on the load index");
+        const int chunk = lpos ^ swz_of_row(wave * RPI + lrow);
+        int ke = chunk * (16 / ES);                 // element index inside K of tile 0
+        cr = ke / (a.KW * a.CI); ke -= cr * (a.KW * a.CI);
+        cs = ke / a.CI; cc = ke - cs * a.CI;
+#pragma unroll
+        for (int i = 0; i < A_LPW; ++i) {
+            const int row = (i * NW + wave) * RPI + lrow;
+            const int m = m0 + row;
+            const int hw = a.HO * a.WO;
+            const int img = m / hw; const int rem = m - img * hw;
+            const int oy = rem / a.WO, ox = rem - oy * a.WO;
+            const bool ok = m < a.M;
+            voffA[i] = (uint32_t)img * (uint32_t)(a.H * a.W * a.CI) * ES;
+            iy0[i] = ok ? oy * a.cstride - a.cpad : -(1 << 28);
+            ix0[i] = ox * a.cstride - a.cpad;
+        }
+    }
+
+    int issue_kt = 0;  // next k-tile to fetch
+    auto issue_tile = [&](int stage) {
+        char* sbase = lds + stage * STAGE_BYTES;
+        const bool live = issue_kt < KT;
+        const bool ragged = (uint32_t)(issue_kt + 1) * BKB > Kb;   // last tile not full (wave-uniform)
+        const uint32_t koff = live ? (uint32_t)issue_kt * BKB : OOB;
+        if constexpr (OP == 0) {
+#pragma unroll
+            for (int i = 0; i < A_LPW; ++i) {
+                uint32_t v = voffA[i] + koff;
+                if (ragged && live) {
+                    const int row = (i * NW + wave) * RPI + lrow;
+                    const uint32_t kb = koff + (uint32_t)((lpos ^ swz_of_row(row)) * 16);
+                    if (kb >= Kb) v = OOB;
+                }
+                load_chunk_to_lds(rsrcA, sbase + (i * NW + wave) * 1024, v);
+            }
+        } else {
+            const int iyr = cr * a.cdil, ixs = cs * a.cdil;
+            const bool kvalid = live && cr < a.KH;
+#pragma unroll
+            for (int i = 0; i < A_LPW; ++i) {
+                const int iy = iy0[i] + iyr, ix = ix0[i] + ixs;
+                const bool ok = kvalid && (unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W;
+                const uint32_t v = ok ? voffA[i] + (uint32_t)((iy * a.W + ix) * a.CI + cc) * ES : OOB;
+                load_chunk_to_lds(rsrcA, sbase + (i * NW + wave) * 1024, v);
+            }
+            // advance the lane's (kh, kw, ci) position by one k-tile
+            cc += BKB / ES;
+            while (cc >= a.CI) { cc -= a.CI; if (++cs == a.KW) { cs = 0; ++cr; } }
+        }
+#pragma unroll
+        for (int i = 0; i < B_LPW; ++i) {
+            uint32_t v = voffB[i] + koff;
+            if (ragged && live) {
+                const int row = (i * NW + wave) * RPI + lrow;
+                const uint32_t kb = koff + (uint32_t)((lpos ^ swz_of_row(row)) * 16);
+                if (kb >= Kb) v = OOB;
+            }
+            load_chunk_to_lds(rsrcB, sbase + A_BYTES + (i * NW + wave) * 1024, v);
+        }
+        ++issue_kt;
+    };
+
+    // ---- per-lane MFMA operand addresses ----
+    const int lr = lane % MT, lq = lane / MT;
+    const int g16 = (lq ^ swz_of_row(lr)) << 4;      // swizzle period <= MT, so only lr matters
+    const int a_lane = (wm_idx * WTM + lr) * BKB;
+    const int b_lane = A_BYTES + (wn_idx * WTN + lr) * BKB;
+
+    acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < ACC_N; ++r) acc[i][j][r] = 0;
+
+    int bsum[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bsum[j] = 0;
+
+    v4i fa[2][TM], fb[2][TN];
+    auto read_frags = [&](int buf, int stage_off, int kk) {
+        const int ko = g16 ^ (kk * KSB);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            fa[buf][i] = *(const v4i*)(lds + stage_off + a_lane + i * MT * BKB + ko);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            fb[buf][j] = *(const v4i*)(lds + stage_off + b_lane + j * MT * BKB + ko);
+    };
+    auto mfma_step = [&](int buf) {
+        if constexpr (DT == 1) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                int s = bsum[j];
+                s = __builtin_amdgcn_sdot4(fb[buf][j].x, 0x01010101, s, false);
+                s = __builtin_amdgcn_sdot4(fb[buf][j].y, 0x01010101, s, false);
+                s = __builtin_amdgcn_sdot4(fb[buf][j].z, 0x01010101, s, false);
+                s = __builtin_amdgcn_sdot4(fb[buf][j].w, 0x01010101, s, false);
+                bsum[j] = s;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            v4i av = fa[buf][i];
+            if constexpr (DT == 1) av = av ^ (int)0x80808080;   // u8 -> s8 by subtracting 128
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = mfma(fb[buf][j], av, acc[i][j]);
+        }
+    };
+
+    // ---- prologue: fill all stages, wait for tile 0 ----
+#pragma unroll
+    for (int s = 0; s < NS; ++s) issue_tile(s);
+    wait_and_barrier<(NS - 1) * LPT, 0>();
+    read_frags(0, 0, 0);
+
+    int stage = 0;
+    for (int kt = 0; kt < KT; ++kt) {
+        const int stage_off = stage * STAGE_BYTES;
+        const int next_stage = (stage + 1 == NS) ? 0 : stage + 1;
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            const int cur = kk & 1;
+            if (kk == KS - 1) {
+                // every fragment of tile kt is in registers: publish tile kt+1, recycle this stage
+                wait_and_barrier<(NS - 2) * LPT, 0>();
+                issue_tile(stage);
+                read_frags(cur ^ 1, next_stage * STAGE_BYTES, 0);
+            } else {
+                read_frags(cur ^ 1, stage_off, kk + 1);
+            }
+            mfma_step(cur);
+            // pin the issue order: fragment reads (and, in the last step, the tile fetch) are
+            // spread between the MFMAs of this step instead of being sunk behind them
+            if (kk == KS - 1) sched_pattern<0, TM + TN, TM * TN, LPT>();
+            else sched_pattern<0, TM + TN, TM * TN, 0>();
+        }
+        stage = next_stage;
+    }
+
+    // ---- epilogue ----
+    // MFMA was issued as (B fragment, A fragment), so a lane holds 4 consecutive n for one m:
+    //   m = lr, n = (r/4)*8 + lq*4 + r%4   (32x32)     m = lr, n = lq*4 + r   (16x16)
+    int* bs_lds = (int*)lds;
+    if constexpr (DT == 1) {
+        // 128 * sum_k B[n,k] completes the u8 x s8 product computed as (u8-128) x s8
+        wait_and_barrier<0, 0>();
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            int s = bsum[j];
+#pragma unroll
+            for (int d = MT; d < 64; d <<= 1) s += __shfl_xor(s, d, 64);
+            if (wm_idx == 0 && lq == 0) bs_lds[wn_idx * WTN + j * MT + lr] = s;
+        }
+        __syncthreads();
+    }
+
+    char* Cb = (char*)a.C + (int64_t)bz * a.sC * OES;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int m = m0 + wm_idx * WTM + i * MT + lr;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int g = 0; g < ACC_N / 4; ++g) {
+                const int nl = wn_idx * WTN + j * MT + g * 8 + lq * 4;
+                const int n = n0 + nl;
+                if (m < a.M && n < a.N) {
+                    char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
+                    if constexpr (DT == 0) {
+                        v4h o;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[i][j][g * 4 + r];
+                        *(v4h*)dst = o;
+                    } else {
+                        const v4i bs = *(const v4i*)(bs_lds + nl);
+                        v4i o;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r] + 128 * bs[r];
+                        *(v4i*)dst = o;
+                    }
+                }
+            }
+        }
+    }
+}

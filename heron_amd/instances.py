@@ -1,0 +1,85 @@
+"""Named template instances that ship pre-compiled (tests, smoke and the benchmark load these).
+
+``precompile`` drives ``hrn_compile`` over a list of descriptors in worker processes; it needs
+hipcc but no GPU, so it runs at build time and the code objects travel with the tree.
+"""
+import os
+from concurrent.futures import ProcessPoolExecutor
+
+from . import backend as B
+
+F16, U8 = B.HRN_DT_F16, B.HRN_DT_U8S8
+GEMM, CONV = B.HRN_OP_GEMM, B.HRN_OP_CONV2D
+
+
+def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0):
+    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe)
+
+
+# (bm, bn, bkb, wm, wn, mfma, stages, swizzle): a spread of the template space used by the parity tests
+PARITY_SHAPES = [
+    (256, 256, 128, 2, 2, 32, 2, 2),
+    (256, 256, 64, 2, 4, 32, 4, 0),
+    (128, 128, 128, 2, 2, 32, 2, 1),
+    (128, 256, 64, 2, 2, 32, 3, 3),
+    (64, 64, 128, 1, 1, 32, 3, 1),
+    (128, 128, 128, 2, 2, 16, 2, 1),
+    (64, 128, 256, 1, 2, 16, 2, 1),
+    (32, 32, 128, 1, 2, 16, 4, 0),
+]
+
+
+def parity_descs():
+    out = []
+    for t in PARITY_SHAPES:
+        out.append(D(F16, GEMM, *t))
+        out.append(D(U8, GEMM, *t))
+    for t in PARITY_SHAPES[:6]:
+        bm, bn, bkb, wm, wn, mfma, st, swz = t
+        if swz and (wm * wn * (64 // (bkb // 16))) % ((bkb // 16) << (swz - 1)):
+            continue
+        out.append(D(F16, CONV, *t))
+    return out
+
+
+# best known instances per benchmark workload (updated from tuning runs)
+BEST = {
+    "gemm_f16": D(F16, GEMM, 256, 256, 128, 2, 2, 32, 2, 2),
+    "gemm_u8s8": D(U8, GEMM, 256, 256, 128, 2, 2, 32, 2, 2),
+    "bmm_f16_qk": D(F16, GEMM, 128, 128, 128, 2, 2, 32, 2, 1),
+    "bmm_f16_pv": D(F16, GEMM, 128, 64, 128, 2, 1, 32, 2, 1),
+    "conv2d_f16": D(F16, CONV, 128, 64, 128, 2, 1, 32, 2, 1),
+    "small": D(U8, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
+    "small_f16": D(F16, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
+}
+
+
+def all_shipped():
+    seen, out = set(), []
+    for d in parity_descs() + list(BEST.values()):
+        if d.as_tuple() not in seen:
+            seen.add(d.as_tuple())
+            out.append(d)
+    return out
+
+
+def _compile_one(tup):
+    d = B.make_desc(*tup)
+    try:
+        return tup, B.compile_desc(d, 300.0), None
+    except Exception as e:  # noqa: BLE001 - reported to the caller
+        return tup, None, str(e)
+
+
+def precompile(descs, jobs=None, verbose=False):
+    """Compile descriptors into the cache with ``jobs`` parallel hipcc workers; returns the failures."""
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    tups = [d.as_tuple() for d in descs]
+    failures = []
+    with ProcessPoolExecutor(max_workers=jobs) as ex:
+        for tup, path, err in ex.map(_compile_one, tups):
+            if err:
+                failures.append((tup, err))
+            if verbose:
+                print(("FAIL " + err[:200]) if err else "ok  ", tup, flush=True)
+    return failures

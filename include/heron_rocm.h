@@ -1,0 +1,176 @@
+/*
+ * heron_rocm.h - C ABI of the MI355X (gfx950) backend for the tensor programs Heron tunes.
+ *
+ * The reference has no FFI of its own for this path: its kernels are generated, built and
+ * timed through TVM from Python.  Each entry point below names the reference interface it
+ * stands in for (paths relative to the reference checkout).  All pointers named A, B, C
+ * are DEVICE pointers owned by the caller; the library never allocates persistent device
+ * memory and never frees caller memory.  Every function returns HRN_OK (0) or a negative
+ * HRN_E_* code; hrn_last_error() gives the message of the last failure on the calling thread.
+ *
+ * Launches are asynchronous on the given stream and may be issued from several host
+ * threads.  The library is NOT fork-safe once a HIP call has been made: processes forked
+ * for sampling must not call into it (hrn_compile is the exception: it never touches HIP).
+ */
+#ifndef HERON_ROCM_H
+#define HERON_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HRN_OK 0
+#define HRN_E_BADPARAM (-1)   /* descriptor/problem violates a template constraint */
+#define HRN_E_BUILD (-2)      /* hipcc failed or timed out */
+#define HRN_E_LOAD (-3)       /* code object could not be loaded */
+#define HRN_E_LAUNCH (-4)     /* HIP reported a launch/runtime error */
+#define HRN_E_TIMEOUT (-5)    /* build exceeded the time limit */
+#define HRN_E_NODEVICE (-6)   /* no HIP device */
+
+/* element types of a template */
+#define HRN_DT_F16 0   /* fp16 x fp16 -> fp32 accumulate -> fp16 store */
+#define HRN_DT_U8S8 1  /* uint8 x int8 -> int32 accumulate -> int32 store */
+
+/* operators */
+#define HRN_OP_GEMM 0    /* C[b,i,j] = sum_k A[b,i,k] * B[b,j,k]  (batch may be 1) */
+#define HRN_OP_CONV2D 1  /* NHWC input, KRSC filter, implicit GEMM */
+
+/*
+ * Device limits the schedule context reads.  Replaces the `check_gpu` dictionary that
+ * the reference's runner hands to its builder (environment.py:110-120, consumed at
+ * schedule/context/cuda_context.py:49-51,74-78).
+ */
+typedef struct hrn_devinfo {
+    char arch[64];            /* e.g. "gfx950:sramecc+:xnack-" */
+    char name[128];
+    int32_t cu_count;
+    int32_t wave_size;
+    int32_t lds_bytes_per_wg;
+    int32_t max_threads_per_wg;
+    int32_t clock_khz;        /* peak engine clock */
+    int32_t mem_clock_khz;
+    int32_t mem_bus_bits;
+    int32_t l2_bytes;
+    int32_t regs_per_simd_lane; /* unified VGPR+AGPR file per lane of one SIMD */
+    int32_t simd_per_cu;
+    uint64_t hbm_bytes;
+} hrn_devinfo;
+
+/*
+ * One instance of the MFMA kernel template = one point of the tuner's search space.
+ * Replaces the (schedule, args) pair the reference gets from Task.instantiate
+ * (task/task.py:76-89) and passes to tvm.build (tests/quick_start/dlboost/run.py:44-46).
+ */
+typedef struct hrn_kernel_desc {
+    int32_t dtype;      /* HRN_DT_* */
+    int32_t op;         /* HRN_OP_* */
+    int32_t bm, bn;     /* workgroup tile (rows of A / rows of B) */
+    int32_t bkb;        /* bytes of K per LDS stage row: 64, 128 or 256 */
+    int32_t wm, wn;     /* wave grid inside the workgroup; waves = wm*wn, 64 lanes each */
+    int32_t mfma;       /* 32 -> 32x32x(16 f16|32 i8), 16 -> 16x16x(32 f16|64 i8) */
+    int32_t stages;     /* LDS stages of the A/B tiles, 2..4 (2 = double buffer) */
+    int32_t swizzle;    /* LDS 16-byte-chunk XOR swizzle: 0 none, 1 row, 2 row/2, 3 row/4 */
+    int32_t epilogue;   /* 0 = store accumulators straight from registers, 1 = stage C through LDS */
+    int32_t waves_per_eu; /* 0 = let the compiler pick, else occupancy hint 1..4 */
+    int32_t reserved[4];
+} hrn_kernel_desc;
+
+/* Resource usage of a built instance, for cross-checks of the constraint set. */
+typedef struct hrn_kernel_info {
+    int32_t vgprs;       /* architectural VGPRs per lane */
+    int32_t agprs;       /* accumulation VGPRs per lane */
+    int32_t sgprs;
+    int32_t lds_bytes;   /* dynamic LDS the launcher requests */
+    int32_t scratch_bytes;
+    int32_t occupancy;   /* waves per SIMD the compiler reports */
+    int32_t threads;     /* workgroup size */
+    int32_t reserved;
+} hrn_kernel_info;
+
+/*
+ * Shapes.  GEMM/bmm: A (batch,M,K), B (batch,N,K), C (batch,M,N), all row-major with the
+ * given leading dimensions (elements) and batch strides (elements).  ops/cuda/dense.py:5-7,
+ * ops/cuda/batch_matmul.py:7-9, ops/x86/dense.py:7-9.
+ * Conv: input (n,h,w,ci), filter (co,kh,kw,ci), output (n,ho,wo,co);
+ * argument order of ops/cuda/conv2d.py:137-139.
+ */
+typedef struct hrn_problem {
+    int32_t op;         /* HRN_OP_* */
+    int32_t batch;
+    int32_t m, n, k;
+    int32_t lda, ldb, ldc;
+    int64_t stride_a, stride_b, stride_c;
+    /* conv only */
+    int32_t cn, ch, cw, ci, co, kh, kw, cstride, cpad, cdil;
+    /* launch-time raster knob: tiles are walked in column groups of this many row-tiles */
+    int32_t group_m;
+    int32_t reserved[3];
+} hrn_problem;
+
+typedef struct hrn_module hrn_module;
+
+/* Device query.  Stands in for runner.get_build_kwargs() (environment.py:110-120). */
+int hrn_device_info(int device, hrn_devinfo* out);
+
+/*
+ * Checks a descriptor against the template's structural constraints without building
+ * (tile divisibility, LDS ceiling, wave count).  Stands in for the feasibility check the
+ * reference leaves to tvm.build failing (runner/measure_methods.py:178-185).
+ */
+int hrn_check_desc(const hrn_kernel_desc* desc);
+
+/*
+ * Compiles one template instance with hipcc into the on-disk cache and returns the path of
+ * the code object.  Touches no GPU (safe in forked/pooled builder processes).  Stands in for
+ * autotvm.LocalBuilder -> tvm.build (tests/quick_start/dlboost/run.py:89-96), including its
+ * `build_timeout` (config.py:48): timeout_s <= 0 means no limit.
+ */
+int hrn_compile(const hrn_kernel_desc* desc, double timeout_s, char* path_out, size_t path_cap);
+
+/* hrn_compile + load on the current device.  Stands in for the module loader of
+ * runner/measure_methods.py:129-130. */
+int hrn_build(const hrn_kernel_desc* desc, double timeout_s, hrn_module** out);
+int hrn_module_info(const hrn_module* mod, hrn_kernel_info* out);
+void hrn_module_free(hrn_module* mod);
+
+/* LDS bytes an instance needs (pure arithmetic; mirrors the constraint of
+ * schedule/context/cuda_context.py:45-63 for this template). */
+int hrn_lds_bytes(const hrn_kernel_desc* desc);
+
+/*
+ * Launchers.  Each replaces the packed function TVM builds for the named operator and that
+ * run.py:60-62 / measure_methods.py:138-145 call with device arrays.
+ *   hrn_launch_gemm_f16        ops/cuda/dense.py:4-54          (fp16 in, fp32 accumulate, fp16 out)
+ *   hrn_launch_gemm_u8s8       ops/x86/dense.py:6-32           (uint8 x int8 -> int32)
+ *   hrn_launch_bmm_f16         ops/cuda/batch_matmul.py:5-56
+ *   hrn_launch_conv2d_nhwc_f16 ops/cuda/conv2d.py:137-232      (filter KRSC)
+ */
+int hrn_launch_gemm_f16(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
+int hrn_launch_gemm_u8s8(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
+int hrn_launch_bmm_f16(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
+int hrn_launch_conv2d_nhwc_f16(const hrn_module* mod, const hrn_problem* p, const void* In, const void* Filter, void* Out, void* stream);
+
+/*
+ * Event-timed measurement with the semantics of TVM's time_evaluator as the reference uses
+ * it (runner/measure_methods.py:138-145): `repeat` results, each the mean seconds of `number`
+ * back-to-back launches; `number` is raised until one repeat lasts at least min_repeat_ms.
+ * costs_out must hold `repeat` doubles.
+ */
+int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C,
+             int number, int repeat, double min_repeat_ms, double* costs_out, void* stream);
+
+/* Fills an hrn_problem for the plain cases (packed row-major operands). */
+void hrn_problem_gemm(hrn_problem* p, int batch, int m, int n, int k);
+void hrn_problem_conv2d(hrn_problem* p, int n, int h, int w, int ci, int co, int kh, int kw,
+                        int stride, int pad, int dil);
+
+const char* hrn_last_error(void);
+const char* hrn_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HERON_ROCM_H */

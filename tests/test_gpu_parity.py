@@ -1,0 +1,186 @@
+"""GPU parity: every shipped template instance against the CPU oracle, through the C ABI.
+
+Integer results must be bit-exact.  fp16 results (fp32 accumulate, one rounding to fp16) must be
+within REL_TOL of the fp32 host reference, measured as max|err| / max|ref| per tensor, plus an
+element-wise check with an fp16-rounding allowance.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from heron_amd import backend as B
+from heron_amd import hostops, instances, workloads
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2          # tolerance stated for fp16 inputs / fp32 accumulate
+_mods = {}
+
+
+def mod_for(desc):
+    key = desc.as_tuple()
+    if key not in _mods:
+        _mods[key] = B.Module(desc)
+    return _mods[key]
+
+
+def dev(a):
+    return torch.from_numpy(a).cuda()
+
+
+def check_f16(got, ref):
+    got = got.astype(np.float32)
+    scale = float(np.abs(ref).max()) + 1e-30
+    err = float(np.abs(got - ref).max())
+    assert err / scale <= REL_TOL, (err, scale)
+    # element-wise: fp16 rounding of the result (2^-11 relative) + accumulation noise
+    assert np.all(np.abs(got - ref) <= 2e-3 * np.abs(ref) + 2e-3 * scale)
+
+
+GEMM_SHAPES = [(64, 64, 64), (256, 256, 256), (512, 640, 384), (100, 200, 72), (8, 4096, 16), (300, 1024, 520)]
+
+
+@pytest.mark.parametrize("tup", instances.PARITY_SHAPES, ids=lambda t: "x".join(map(str, t)))
+def test_gemm_u8s8_bit_exact(tup, hrn):
+    m = mod_for(instances.D(instances.U8, instances.GEMM, *tup))
+    for i, (M, K, N) in enumerate(GEMM_SHAPES):
+        K16 = (K + 15) // 16 * 16
+        A, Bm = workloads.gemm_u8s8_inputs(M, K16, N, seed=10 + i)
+        print("u8s8", tup, (M, K16, N), flush=True)
+        C = hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy()
+        ref = oracle.gemm_u8s8s32_dlboost(A, Bm) if N % 32 == 0 else oracle.gemm_int64_numpy(A, Bm).astype(np.int32)
+        assert np.array_equal(C, ref)
+
+
+@pytest.mark.parametrize("tup", instances.PARITY_SHAPES, ids=lambda t: "x".join(map(str, t)))
+def test_gemm_f16_within_tolerance(tup, hrn):
+    m = mod_for(instances.D(instances.F16, instances.GEMM, *tup))
+    for i, (M, K, N) in enumerate(GEMM_SHAPES):
+        K8 = (K + 7) // 8 * 8
+        A, Bm = workloads.gemm_f16_inputs(M, K8, N, seed=20 + i, scale=1.0 if i % 2 else 0.1)
+        print("f16", tup, (M, K8, N), flush=True)
+        C = hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy()
+        check_f16(C, oracle.gemm_f32(A, Bm))
+
+
+def test_gemm_u8s8_extremes(hrn):
+    """A = 255, B = -128 reaches the most negative accumulator; B = 127 the most positive."""
+    m = mod_for(instances.BEST["small"])
+    M = N = 64
+    for K in (64, 4096, 8192):
+        A = np.full((M, K), 255, np.uint8)
+        for bv in (-128, 127):
+            Bm = np.full((N, K), bv, np.int8)
+            C = hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy()
+            assert np.all(C == 255 * bv * K)
+        # identity-like B picks single columns of A
+        A2, _ = workloads.gemm_u8s8_inputs(M, K, N, seed=K)
+        Bm = np.zeros((N, K), np.int8)
+        Bm[np.arange(N), np.arange(N)] = 1
+        C = hostops.gemm(m, dev(A2), dev(Bm)).cpu().numpy()
+        assert np.array_equal(C, A2[:, :N].astype(np.int32))
+
+
+def test_gemm_f16_exact_cases(hrn):
+    """Power-of-two scaling is exact; integer-valued inputs with small sums are exact in fp16."""
+    m = mod_for(instances.BEST["small_f16"])
+    rng = np.random.default_rng(7)
+    A = rng.integers(-4, 5, (96, 64)).astype(np.float16)
+    Bm = rng.integers(-4, 5, (80, 64)).astype(np.float16)
+    C = hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy()
+    ref = (A.astype(np.int64) @ Bm.astype(np.int64).T)
+    assert np.array_equal(C.astype(np.int64), ref)          # |sum| <= 1024 < 2048: exact in fp16
+    C4 = hostops.gemm(m, dev((A * 4).astype(np.float16)), dev(Bm)).cpu().numpy()
+    assert np.array_equal(C4, C * 4)
+
+
+@pytest.mark.parametrize("tup", instances.PARITY_SHAPES[:5], ids=lambda t: "x".join(map(str, t)))
+def test_bmm_f16(tup, hrn):
+    m = mod_for(instances.D(instances.F16, instances.GEMM, *tup))
+    for (b, M, K, N) in [(3, 128, 64, 192), (5, 72, 128, 40)]:
+        Q, Kt = workloads.bmm_qk_inputs(b, M, K, N, seed=b)
+        print("bmm", tup, (b, M, K, N), flush=True)
+        C = hostops.gemm(m, dev(Q), dev(Kt)).cpu().numpy()
+        check_f16(C, oracle.bmm_f32(Q, Kt))
+        # batch independence: a permuted batch gives the permuted result, bit for bit
+        perm = np.roll(np.arange(b), 1)
+        Cp = hostops.gemm(m, dev(Q[perm].copy()), dev(Kt[perm].copy())).cpu().numpy()
+        assert np.array_equal(Cp, C[perm])
+    P, Vt = workloads.bmm_pv_inputs(2, 64, 128, 64, seed=3)
+    ones = np.ones((2, 8, 128), np.float16)
+    R = hostops.gemm(m, dev(P), dev(ones)).cpu().numpy()     # rows of P sum to 1
+    assert np.abs(R.astype(np.float32) - 1).max() < 5e-3
+
+
+def test_bmm_u8s8(hrn):
+    m = mod_for(instances.BEST["small"])
+    rng = np.random.default_rng(11)
+    A = rng.integers(0, 256, (4, 96, 80), dtype=np.uint8)
+    Bm = rng.integers(-128, 128, (4, 72, 80), dtype=np.int8)
+    C = hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy()
+    assert np.array_equal(C, oracle.bmm_u8s8s32_scalar(A, Bm))
+
+
+CONV_CASES = [
+    # N, H, W, CI, CO, KH, KW, stride, pad, dil
+    (2, 14, 14, 64, 64, 3, 3, 1, 1, 1),
+    (1, 9, 11, 16, 32, 3, 3, 1, 1, 1),
+    (2, 8, 8, 32, 48, 1, 1, 1, 0, 1),
+    (1, 15, 15, 8, 16, 3, 3, 2, 1, 1),
+    (1, 12, 12, 24, 8, 3, 3, 1, 2, 2),
+    (3, 7, 7, 128, 64, 5, 5, 1, 2, 1),
+]
+
+
+def _conv_tuples():
+    return [d.as_tuple()[2:10] for d in instances.parity_descs() if d.op == instances.CONV]
+
+
+@pytest.mark.parametrize("tup", _conv_tuples(), ids=lambda t: "x".join(map(str, t)))
+def test_conv2d_nhwc_f16(tup, hrn):
+    m = mod_for(instances.D(instances.F16, instances.CONV, *tup))
+    for i, (N, H, W, CI, CO, KH, KW, s, p, d) in enumerate(CONV_CASES):
+        X, Wt = workloads.conv2d_inputs(N, H, W, CI, CO, KH, KW, seed=30 + i)
+        print("conv", tup, CONV_CASES[i], flush=True)
+        Y = hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, d).cpu().numpy()
+        check_f16(Y, oracle.conv2d_nhwc_f32(X, Wt, s, p, d))
+
+
+def test_conv_1x1_is_gemm(hrn):
+    """A 1x1 convolution is the GEMM of the flattened pixels: both templates must agree bit for bit."""
+    tup = instances.PARITY_SHAPES[2]
+    mc = mod_for(instances.D(instances.F16, instances.CONV, *tup))
+    mg = mod_for(instances.D(instances.F16, instances.GEMM, *tup))
+    X, Wt = workloads.conv2d_inputs(2, 8, 8, 64, 64, 1, 1, seed=5)
+    Y = hostops.conv2d_nhwc(mc, dev(X), dev(Wt)).cpu().numpy()
+    G = hostops.gemm(mg, dev(X.reshape(-1, 64)), dev(Wt.reshape(64, 64))).cpu().numpy()
+    assert np.array_equal(Y.reshape(-1, 64), G)
+
+
+def test_error_paths(hrn):
+    """Bad descriptors and problems come back as error codes, not as launches."""
+    bad = instances.D(instances.F16, instances.GEMM, 256, 256, 128, 2, 2, 32, 3, 2)   # 192 KiB of LDS
+    assert not B.check_desc(bad)
+    with pytest.raises(B.HeronRocmError):
+        B.Module(bad)
+    m = mod_for(instances.BEST["small_f16"])
+    A = torch.zeros((64, 60), dtype=torch.float16, device="cuda")       # K*2 not a multiple of 16
+    with pytest.raises(B.HeronRocmError):
+        hostops.gemm(m, A, A)
+    mu = mod_for(instances.BEST["small"])
+    with pytest.raises(ValueError):
+        hostops.gemm(mu, A, A)                                           # wrong dtype for the module
+
+
+def test_device_info_and_timing(hrn):
+    info = B.device_info(0)
+    assert info["arch"].startswith("gfx950") and info["wave_size"] == 64 and info["cu_count"] > 0
+    m = mod_for(instances.BEST["small_f16"])
+    A, Bm = workloads.gemm_f16_inputs(256, 256, 256)
+    a, b = dev(A), dev(Bm)
+    c = torch.empty((256, 256), dtype=torch.float16, device="cuda")
+    costs = m.time(B.gemm_problem(1, 256, 256, 256), a.data_ptr(), b.data_ptr(), c.data_ptr(), number=3, repeat=4,
+                   min_repeat_ms=1.0)
+    assert len(costs) == 4 and all(0 < x < 1e-2 for x in costs)
+    check_f16(c.cpu().numpy(), oracle.gemm_f32(A, Bm))
