@@ -1,0 +1,204 @@
+"""Benchmark of the MFMA hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+One step = one launch of the tuned template instance over a batch of synthetic operands that are
+already resident in HBM.  Prints ONE JSON line.  The headline workload is the dense fp16 GEMM
+M=N=K=4096 (fp32 accumulate, fp16 output); the other benchmark configurations are reported under
+"also" in the same line.  `roofline.achieved` is algorithmic work per launch divided by the average
+kernel duration measured with HIP events on the launch stream.  `cpu_baseline` times the CPU oracle
+(the DL Boost-style VNNI GEMM for the quantized case, the fp32 host reference otherwise) on a bounded
+sample of the same workload, on this machine's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def make_workloads(torch, workloads, instances):
+    """name -> dict(desc, problem factory, device operands, ops, bytes, peak, dtype)."""
+    from heron_amd import backend as B
+
+    def dev(a):
+        return torch.from_numpy(a).cuda()
+
+    W = {}
+
+    def add_gemm(name, key, M, K, N, f16, batch=1, gen=None, group_m=8):
+        def build():
+            if gen is not None:
+                A, Bm = gen()
+            elif f16:
+                A, Bm = workloads.gemm_f16_inputs(M, K, N, seed=1)
+            else:
+                A, Bm = workloads.gemm_u8s8_inputs(M, K, N, seed=2)
+            shape = (batch, M, N) if batch > 1 else (M, N)
+            C = torch.empty(shape, dtype=torch.float16 if f16 else torch.int32, device="cuda")
+            return dev(A), dev(Bm), C, B.gemm_problem(batch, M, N, K, group_m)
+        ops, byts = workloads.gemm_work(M, N, K, 2 if f16 else 1, 2 if f16 else 4, batch)
+        W[name] = dict(desc=instances.BEST[key], build=build, ops=ops, bytes=byts, f16=f16,
+                       desc_text="%s batch=%d M=%d N=%d K=%d" % ("gemm_f16" if f16 else "gemm_u8s8", batch, M, N, K))
+
+    add_gemm("gemm_f16_4096", "gemm_f16", 4096, 4096, 4096, True)
+    add_gemm("gemm_f16_8192", "gemm_f16", 8192, 8192, 8192, True)
+    add_gemm("gemm_u8s8_8192", "gemm_u8s8", 8192, 8192, 8192, False)
+    add_gemm("bmm_f16_qk", "bmm_f16_qk", 512, 64, 512, True, 192, lambda: workloads.bmm_qk_inputs(192, 512, 64, 512))
+    add_gemm("bmm_f16_pv", "bmm_f16_pv", 512, 512, 64, True, 192, lambda: workloads.bmm_pv_inputs(192, 512, 512, 64))
+
+    def build_conv():
+        X, Wt = workloads.conv2d_inputs(32, 56, 56, 64, 64, 3, 3, seed=3)
+        Y = torch.empty((32, 56, 56, 64), dtype=torch.float16, device="cuda")
+        return dev(X), dev(Wt), Y, B.conv2d_problem(32, 56, 56, 64, 64, 3, 3, 1, 1, 1, 8)
+    ops, byts = workloads.conv_work(32, 56, 56, 64, 64, 3, 3, 1, 1, 1)
+    W["conv2d_f16_resnet"] = dict(desc=instances.BEST["conv2d_f16"], build=build_conv, ops=ops, bytes=byts, f16=True,
+                                  desc_text="conv2d_nhwc_f16 N=32 H=W=56 C=64 K=64 3x3 s1 p1")
+    return W
+
+
+def measure(torch, B, w, steps, warmup):
+    """Returns (wall seconds per step, event seconds per launch)."""
+    mod = B.Module(w["desc"])
+    a, b, c, prob = w["build"]()
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(warmup):
+        mod.launch(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        mod.launch(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), stream)
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    # per-launch kernel duration from HIP events recorded on the launch stream
+    costs = mod.time(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), number=steps, repeat=3, min_repeat_ms=0.0, stream=stream)
+    ev = sorted(costs)[len(costs) // 2]
+    info = dict(mod.info)
+    mod.close()
+    del a, b, c
+    return wall, ev, info
+
+
+def roofline(w, ev_seconds, workloads):
+    ai = w["ops"] / w["bytes"]
+    peak_mfma = workloads.PEAK_FP16_TFLOPS if w["f16"] else workloads.PEAK_INT8_TOPS
+    ridge = peak_mfma * 1e12 / (workloads.PEAK_HBM_GBS * 1e9)
+    if ai >= ridge:
+        ach = w["ops"] / ev_seconds / 1e12
+        return {"bound": "mfma", "achieved": ach, "peak": peak_mfma, "unit": "TFLOP/s" if w["f16"] else "TOP/s",
+                "frac": ach / peak_mfma, "traffic": None}
+    ach = w["bytes"] / ev_seconds / 1e9
+    return {"bound": "hbm", "achieved": ach, "peak": workloads.PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": ach / workloads.PEAK_HBM_GBS, "traffic": None}
+
+
+def cpu_baseline(name, workloads):
+    """The CPU oracle on a bounded sample of the workload (checker code used as a reported baseline only)."""
+    import numpy as np
+    import oracle
+    cores = len(os.sched_getaffinity(0))
+    if name.startswith("gemm_u8s8"):
+        M, K, N = 8192, 8192, 8192
+        A, Bm = workloads.gemm_u8s8_inputs(M, K, N, seed=2)
+        if oracle.has_vnni():
+            pb = oracle.PackedB(Bm)
+            C = np.empty((M, N), np.int32)
+            pb.matmul(A[:256], out=C[:256])                # warm-up
+            reps, t0 = 0, time.perf_counter()
+            while True:
+                pb.matmul(A, out=C)
+                reps += 1
+                if time.perf_counter() - t0 > 10 or reps >= 20:
+                    break
+            dt = (time.perf_counter() - t0) / reps
+            return {"value": 2.0 * M * N * K / dt / 1e12, "unit": "TOP/s", "cores": oracle.num_threads(), "kind": "port",
+                    "sample": "full 8192^3 u8s8 GEMM x%d, AVX512-VNNI 16x4 vpdpbusd micro-kernel, B pre-packed, "
+                              "%d OpenMP threads of %d host cores" % (reps, oracle.num_threads(), cores)}
+        rows = 64
+        t0 = time.perf_counter()
+        oracle.gemm_u8s8s32_dlboost(A[:rows], Bm)
+        dt = time.perf_counter() - t0
+        return {"value": 2.0 * rows * N * K / dt / 1e12, "unit": "TOP/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": "%d rows of the 8192^3 u8s8 GEMM, scalar fallback (no AVX512-VNNI)" % rows}
+    # fp16 workloads: fp32 host reference (double accumulate) on a slab of rows
+    M, K, N = 4096, 4096, 4096
+    A, Bm = workloads.gemm_f16_inputs(M, K, N, seed=1)
+    rows = 64
+    Af, Bf = A[:rows].astype(np.float32), Bm.astype(np.float32)
+    oracle.gemm_f32(Af[:8], Bf)
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        oracle.gemm_f32(Af, Bf)
+        reps += 1
+        if time.perf_counter() - t0 > 10 or reps >= 50:
+            break
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": 2.0 * rows * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": "%d of 4096 rows of the fp16 GEMM 4096^3 x%d, fp32 host reference (double accumulate), "
+                      "%d OpenMP threads of %d host cores" % (rows, reps, oracle.num_threads(), cores)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="gemm_f16_4096")
+    ap.add_argument("--only", action="store_true", help="skip the 'also' workloads and the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the hot path is a single-GPU kernel and no multi-GPU figure is produced "
+              "(got --gpus %d)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from heron_amd import backend as B
+    from heron_amd import instances, workloads
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    B.lib()
+    W = make_workloads(torch, workloads, instances)
+    if args.workload not in W:
+        print("unknown workload %s (have %s)" % (args.workload, sorted(W)), file=sys.stderr)
+        sys.exit(2)
+
+    w = W[args.workload]
+    wall, ev, info = measure(torch, B, w, args.steps, args.warmup)
+    line = {
+        "metric": "%s throughput per GPU (tuned MFMA template)" % ("fp16 GEMM TFLOPS" if w["f16"] else "u8s8 GEMM TOPS"),
+        "value": w["ops"] / wall / 1e12,
+        "unit": "TFLOP/s" if w["f16"] else "TOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16" if w["f16"] else "u8",
+        "data": "synthetic",
+        "config": {"workload": w["desc_text"], "instance": repr(w["desc"]), "kernel_ms": ev * 1e3, "resources": info},
+        "roofline": roofline(w, ev, workloads),
+    }
+    if not args.only:
+        also = []
+        for name, ww in W.items():
+            if name == args.workload:
+                continue
+            steps = max(10, min(args.steps, 50))
+            wl, e, _ = measure(torch, B, ww, steps, min(args.warmup, 5))
+            r = roofline(ww, e, workloads)
+            also.append({"workload": ww["desc_text"], "value": ww["ops"] / wl / 1e12,
+                         "unit": "TFLOP/s" if ww["f16"] else "TOP/s", "kernel_ms": e * 1e3,
+                         "frac_of_mfma_peak": ww["ops"] / e / 1e12 / (workloads.PEAK_FP16_TFLOPS if ww["f16"] else workloads.PEAK_INT8_TOPS),
+                         "roofline": r})
+        line["also"] = also
+        line["cpu_baseline"] = cpu_baseline(args.workload, workloads)
+        line["cpu_baseline_u8s8"] = cpu_baseline("gemm_u8s8_8192", workloads) if not args.workload.startswith("gemm_u8s8") else None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

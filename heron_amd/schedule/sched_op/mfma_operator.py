@@ -1,0 +1,337 @@
+"""Schedule operations of the MFMA kernel template, and the CDNA4 constraint set.
+
+In the reference a schedule operation transforms TVM loops and, while the template is being
+built, registers the knobs and constraints the transformation implies
+(schedule/sched_op/sched_common.py, gpu_common.py, gpu_tensorcore_operator.py).  Here the kernel is
+a fixed hand-written HIP template, so an operation only (a) registers knobs/constraints in
+building mode and (b) copies the solved values into the ``TemplateSchedule``; replaying
+``knob_manager.sched_tups`` with a solved KnobManager therefore yields a concrete template
+instance, exactly as ``Task.instantiate`` replays TVM primitives in the reference.
+
+Each constraint cites the reference constraint it replaces.
+"""
+from ...utils import genKey
+
+
+class TemplateSchedule:
+    """What ``te.create_schedule`` is to the reference: the object the operations fill in."""
+
+    def __init__(self, outs, info):
+        self.outs = outs
+        self.info = info
+        self.params = {}
+
+    def __getitem__(self, key):
+        return self.params[key]
+
+    def to_desc(self):
+        from ... import backend as B
+        p = self.params
+        dtype = B.HRN_DT_F16 if self.info['kind'] == 'f16' else B.HRN_DT_U8S8
+        op = B.HRN_OP_CONV2D if self.info['operator'] == 'conv2d_nhwc' else B.HRN_OP_GEMM
+        return B.make_desc(dtype, op, p['bm'], p['bn'], p['bkb'], p['wm'], p['wn'], p['mfma'], p['stages'],
+                           p['swizzle'], 0, p['waves_per_eu'])
+
+    def to_problem(self):
+        from ... import backend as B
+        g = self.info['gemm_view']
+        if self.info['operator'] == 'conv2d_nhwc':
+            c = self.info['conv']
+            return B.conv2d_problem(c['N'], c['H'], c['W'], c['CI'], c['CO'], c['KH'], c['KW'], c['stride'],
+                                    c['pad'], c['dil'], self.params['group_m'])
+        return B.gemm_problem(g['batch'], g['M'], g['N'], g['K'], self.params['group_m'])
+
+    def describe(self):
+        return ", ".join("%s=%s" % kv for kv in sorted(self.params.items()))
+
+
+def roundup(x, m):
+    return (x + m - 1) // m * m
+
+
+class schedOp:
+    def __init__(self, name):
+        self.name = name
+
+    # --- helpers -----------------------------------------------------------------------
+    @staticmethod
+    def P(stage, param):
+        return genKey("P", stage, param_name=param)
+
+    @staticmethod
+    def V(stage, var):
+        return genKey("V", stage, var_name=var)
+
+    @staticmethod
+    def L(stage, ax):
+        return genKey("L", stage, ax)
+
+    def knob(self, ctx, stage, param, candidates, default):
+        """A tunable parameter restricted to ``candidates`` (the define_knob + addCandidates idiom of
+        gpu_tensorcore_operator.py:285-294)."""
+        km = ctx.knob_manager
+        key = self.P(stage, param)
+        km.define_value(key, min(candidates), max(candidates), default, True)
+        if list(candidates) != list(range(min(candidates), max(candidates) + 1)):
+            km.addCandidates(key, list(candidates))
+        else:
+            km.addRawCandidates(key, list(candidates))
+        return key
+
+    def var(self, ctx, stage, name, low, up, default=None):
+        return ctx.knob_manager.define_value(self.V(stage, name), low, up, low if default is None else default)
+
+    def perform(self, s, stage_name, ctx):
+        raise NotImplementedError
+
+
+class startOp(schedOp):
+    """Declares the GEMM view of the stage as loop extents (the role of startOp in sched_common.py:
+    axis extents enter the CSP as constants)."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        g, kind = s.info['gemm_view'], s.info['kind']
+        es = 2 if kind == 'f16' else 1
+        # spatial extents are padded to one 16-row MFMA tile, K (in bytes) to one 64-byte LDS row
+        km.axis_ori_lenth[self.L(stage_name, 'i')] = roundup(g['M'], 16)
+        km.axis_ori_lenth[self.L(stage_name, 'j')] = roundup(g['N'], 16)
+        km.axis_ori_lenth[self.L(stage_name, 'k')] = roundup(g['K'] * es, 64)
+        km.axis_ori_lenth[self.L(stage_name, 'b')] = g['batch']
+        ctx.addSchedDesc("\n## Stage %s: %s %s, GEMM view batch=%d M=%d N=%d K=%d\n" % (
+            stage_name, s.info['operator'], kind, g['batch'], g['M'], g['N'], g['K']))
+
+
+class mfmaShapeOp(schedOp):
+    """MFMA instruction shape: 32x32x(16 f16 | 32 i8) or 16x16x(32 f16 | 64 i8); both consume 1024
+    operand bytes per wave.  Replaces the wmma m/n/k candidates [8,16,32] with m*n*k = 4096
+    (gpu_tensorcore_operator.py:285-294)."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        mfma = self.knob(ctx, stage_name, 'mfma', [16, 32], 32)
+        ksb = self.var(ctx, stage_name, 'mfma_k_bytes', 32, 64, 32)
+        km.addProd([mfma, ksb], 1024)
+        m2 = self.var(ctx, stage_name, 'mfma_area', 256, 1024, 1024)
+        km.addProd([mfma, mfma], m2)
+        apt = self.var(ctx, stage_name, 'acc_regs_per_tile', 4, 16, 16)
+        km.addProd([64, apt], m2)                     # one accumulator register per 64 outputs
+        s.params['mfma'] = km.get_val(mfma)
+        ctx.addSchedDesc("mfma = %s  # %s\n" % (km.get_val(mfma), mfma))
+
+
+class tileWaveOp(schedOp):
+    """Wave grid and per-wave MFMA tiling: lanes per wave are fixed at 64 (replaces
+    addEQ(threadIdx.x, 32), gpu_common.py:36-37) and waves = wm*wn <= max_threads/64 (replaces
+    threads <= 1024, cuda_context.py:25-32)."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        max_waves = ctx.getLimit('max_threads_per_wg') // ctx.getLimit('wave_size')
+        wm = self.knob(ctx, stage_name, 'wave_m', [1, 2, 4, 8], 2)
+        wn = self.knob(ctx, stage_name, 'wave_n', [1, 2, 4, 8], 2)
+        waves = self.var(ctx, stage_name, 'waves', 1, max_waves, 4)
+        km.addProd([wm, wn], waves)
+        tm = self.knob(ctx, stage_name, 'tile_m', list(range(1, 9)), 2)
+        tn = self.knob(ctx, stage_name, 'tile_n', list(range(1, 9)), 2)
+        mfma = self.P(stage_name, 'mfma')
+        wtm = self.var(ctx, stage_name, 'wave_tile_m', 16, 256, 64)
+        wtn = self.var(ctx, stage_name, 'wave_tile_n', 16, 256, 64)
+        km.addProd([tm, mfma], wtm)
+        km.addProd([tn, mfma], wtn)
+        for k, key in (('wm', wm), ('wn', wn), ('tm', tm), ('tn', tn)):
+            s.params[k] = km.get_val(key)
+        ctx.addSchedDesc("wave grid = %s x %s, mfma tiles per wave = %s x %s\n" % tuple(
+            km.get_val(k) for k in (wm, wn, tm, tn)))
+
+
+class tileBlockOp(schedOp):
+    """Workgroup tile: M = grid_m * bm, bm = wm * wave_tile_m (and the same for N), the ProdTwo chain of
+    a two-level split (knobManager.py:83-107)."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        for ax, w, wt, b, g in (('i', 'wave_m', 'wave_tile_m', 'block_m', 'grid_m'),
+                                ('j', 'wave_n', 'wave_tile_n', 'block_n', 'grid_n')):
+            extent = km.axis_ori_lenth[self.L(stage_name, ax)]
+            bkey = self.var(ctx, stage_name, b, 16, min(512, extent), 16)
+            gkey = self.var(ctx, stage_name, g, 1, extent // 16, extent // 16)
+            km.addProd([self.P(stage_name, w), self.V(stage_name, wt)], bkey)
+            km.addProd([gkey, bkey], extent)
+            s.params['bm' if ax == 'i' else 'bn'] = km.get_val(bkey)
+        ctx.addSchedDesc("block tile = %s x %s\n" % (s.params['bm'], s.params['bn']))
+
+
+class tileKOp(schedOp):
+    """K tiling: bkb bytes of K per LDS row, an even number >= 2 of MFMA k-steps per tile, and K an exact
+    multiple of the tile (the split constraint of the reduce axis, sched_common.py generalTileOp)."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        kbytes = km.axis_ori_lenth[self.L(stage_name, 'k')]
+        bkb = self.knob(ctx, stage_name, 'block_k_bytes', [64, 128, 256], 128)
+        ks = self.var(ctx, stage_name, 'k_steps', 2, 8, 4)
+        km.addCandidates(ks, [2, 4, 8])
+        km.addProd([ks, self.V(stage_name, 'mfma_k_bytes')], bkb)
+        kt = self.var(ctx, stage_name, 'k_tiles', 1, kbytes // 64, kbytes // 64)
+        km.addProd([kt, bkb], kbytes)
+        s.params['bkb'] = km.get_val(bkb)
+        ctx.addSchedDesc("k tile = %s bytes\n" % s.params['bkb'])
+
+
+class loadVectorOp(schedOp):
+    """Global->LDS transfer: every lane moves one 128-bit chunk per load and one wave instruction fills
+    1 KiB of LDS, so a tile must split into whole wave loads: bm = loads_a * (64/chunks_per_row) * waves.
+    Replaces the vectorize candidates [1,2,4,8] halfs and their stride filter
+    (gpu_tensorcore_operator.py:15-21): the width is fixed at 16 bytes, the divisibility is what remains."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        bkb = self.P(stage_name, 'block_k_bytes')
+        cpr = self.var(ctx, stage_name, 'chunks_per_row', 4, 16, 8)
+        km.addProd([16, cpr], bkb)
+        rpi = self.var(ctx, stage_name, 'rows_per_load', 4, 16, 8)
+        km.addProd([rpi, cpr], 64)
+        rpr = self.var(ctx, stage_name, 'rows_per_round', 4, 256, 32)
+        km.addProd([rpi, self.V(stage_name, 'waves')], rpr)
+        la = self.var(ctx, stage_name, 'loads_a', 1, 32, 1)
+        lb = self.var(ctx, stage_name, 'loads_b', 1, 32, 1)
+        km.addProd([la, rpr], self.V(stage_name, 'block_m'))
+        km.addProd([lb, rpr], self.V(stage_name, 'block_n'))
+        lpt = self.var(ctx, stage_name, 'loads_per_tile', 2, 64, 2)
+        km.addSUM(lpt, [la, lb])
+        ctx.addSchedDesc("global->LDS: 16-byte chunks, direct to LDS\n")
+
+
+class ldsStageOp(schedOp):
+    """LDS staging: stages * (bm + bn) * bkb <= LDS bytes per workgroup (replaces shared_mem_size <=
+    max_shared_memory_per_block/2 elements, cuda_context.py:45-63), and the loads in flight
+    (stages-1) * loads_per_tile must fit the 6-bit vmcnt counter."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        lds_limit = ctx.getLimit('lds_bytes_per_wg')
+        stages = self.knob(ctx, stage_name, 'lds_stages', [2, 3, 4], 2)
+        bmn = self.var(ctx, stage_name, 'block_m_plus_n', 32, 1024, 32)
+        km.addSUM(bmn, [self.V(stage_name, 'block_m'), self.V(stage_name, 'block_n')])
+        sb = self.var(ctx, stage_name, 'stage_bytes', 2048, lds_limit // 2, 2048)
+        km.addProd([bmn, self.P(stage_name, 'block_k_bytes')], sb)
+        lds = self.var(ctx, stage_name, 'lds_bytes', 4096, lds_limit, 4096)
+        km.addProd([stages, sb], lds)
+        if lds not in km.mems:
+            km.mems.append(lds)
+        ahead = self.var(ctx, stage_name, 'stages_ahead', 1, 3, 1)
+        km.addSUM(stages, [ahead, 1])
+        inflight = self.var(ctx, stage_name, 'loads_in_flight', 1, ctx.getLimit('max_loads_in_flight'), 1)
+        km.addProd([ahead, self.V(stage_name, 'loads_per_tile')], inflight)
+        s.params['stages'] = km.get_val(stages)
+        ctx.addSchedDesc("LDS stages = %s\n" % s.params['stages'])
+
+
+class ldsSwizzleOp(schedOp):
+    """XOR swizzle of the 16-byte chunks of an LDS row with (row >> (swizzle-1)); its period
+    chunks_per_row << (swizzle-1) must not exceed the MFMA tile edge.  Replaces the storage_align
+    offsets [0,8,16,24,32,48] (gpu_common.py:133-152): padding is impossible with direct-to-LDS
+    loads (one instruction writes 1 KiB contiguously), swizzling does the same job."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        swz = self.knob(ctx, stage_name, 'lds_swizzle', [0, 1, 2, 3], 1)
+        cpr = self.V(stage_name, 'chunks_per_row')
+        p2 = self.var(ctx, stage_name, 'swizzle_period2', 8, 32, 16)
+        p4 = self.var(ctx, stage_name, 'swizzle_period4', 16, 64, 32)
+        km.addProd([2, cpr], p2)
+        km.addProd([4, cpr], p4)
+        period = self.var(ctx, stage_name, 'swizzle_period', 1, 32, 8)
+        km.addSelect([1, cpr, p2, p4], swz, period)
+        km.addLE(period, self.P(stage_name, 'mfma'))
+        if s.info['operator'] == 'conv2d_nhwc':
+            # the lane's chunk column must be the same for every load of a tile
+            q = self.var(ctx, stage_name, 'rounds_per_period', 1, 256, 1)
+            km.addProd([q, period], self.V(stage_name, 'rows_per_round'))
+        s.params['swizzle'] = km.get_val(swz)
+        ctx.addSchedDesc("LDS swizzle = %s\n" % s.params['swizzle'])
+
+
+class registerBudgetOp(schedOp):
+    """Register file: accumulators tm*tn*(mfma^2/64) <= 256 per lane, plus double-buffered operand
+    fragments 8*(tm+tn) and a fixed allowance for addresses; times the waves each SIMD hosts
+    (waves/4, at least 1) it must fit the 512-entry unified VGPR+AGPR file.  No counterpart in the
+    reference (NVCC allocates registers behind TVM's back)."""
+
+    OVERHEAD = 48
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        regs_total = ctx.getLimit('regs_per_simd_lane')
+        simds = ctx.getLimit('simd_per_cu')
+        tm, tn = self.P(stage_name, 'tile_m'), self.P(stage_name, 'tile_n')
+        tmn = self.var(ctx, stage_name, 'tiles_per_wave', 1, 64, 4)
+        km.addProd([tm, tn], tmn)
+        acc = self.var(ctx, stage_name, 'acc_regs', 4, regs_total // 2, 64)
+        km.addProd([tmn, self.V(stage_name, 'acc_regs_per_tile')], acc)
+        tsum = self.var(ctx, stage_name, 'tile_m_plus_n', 2, 16, 4)
+        km.addSUM(tsum, [tm, tn])
+        frag = self.var(ctx, stage_name, 'frag_regs', 16, 128, 32)
+        km.addProd([8, tsum], frag)
+        regs = self.var(ctx, stage_name, 'regs_per_lane', 1, regs_total, 128)
+        km.addSUM(regs, [acc, frag, self.OVERHEAD])
+        # waves of one workgroup that share a SIMD
+        waves = self.V(stage_name, 'waves')
+        wps = self.var(ctx, stage_name, 'waves_per_simd', 1, 4, 1)
+        max_waves = ctx.getLimit('max_threads_per_wg') // ctx.getLimit('wave_size')
+        cands = [w for w in (1, 2, 4, 8, 16) if w <= max_waves]
+        km.addCandidates(waves, cands)
+        from ..constraints.primitives import EQ
+        if km.is_building:
+            for idx, w in enumerate(cands):
+                km.solver.primitives.append(EQ([wps, max(1, w // simds)], cond="O#" + waves + '_cand%d' % idx))
+        budget = self.var(ctx, stage_name, 'regs_per_simd', 1, regs_total, 128)
+        km.addProd([regs, wps], budget)
+        hint = self.knob(ctx, stage_name, 'waves_per_eu', [0, 1, 2], 0)
+        hinted = self.var(ctx, stage_name, 'regs_hinted', 0, regs_total, 0)
+        km.addProd([hint, regs], hinted)
+        s.params['waves_per_eu'] = km.get_val(hint)
+        ctx.addSchedDesc("occupancy hint = %s\n" % s.params['waves_per_eu'])
+
+
+class rasterOp(schedOp):
+    """Launch-time tile raster: workgroups are spread over the 8 XCDs and walk the tile grid in column
+    groups of ``group_m`` row-tiles so that one XCD's L2 holds a compact block of A and B."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        gm = self.knob(ctx, stage_name, 'raster_group_m', [1, 2, 4, 8, 16, 32], 8)
+        s.params['group_m'] = km.get_val(gm)
+        ctx.addSchedDesc("raster group_m = %s\n" % s.params['group_m'])
+
+
+class finishOp(schedOp):
+    def perform(self, s, stage_name, ctx):
+        ctx.addSchedDesc("# template instance: %s\n" % s.describe())
+
+
+all_op_methods = {
+    'start': startOp,
+    'mfmaShape': mfmaShapeOp,
+    'tileWave': tileWaveOp,
+    'tileBlock': tileBlockOp,
+    'tileK': tileKOp,
+    'loadVector': loadVectorOp,
+    'ldsStage': ldsStageOp,
+    'ldsSwizzle': ldsSwizzleOp,
+    'registerBudget': registerBudgetOp,
+    'raster': rasterOp,
+    'finish': finishOp,
+}
+
+RULE_ORDER = ['start', 'mfmaShape', 'tileWave', 'tileBlock', 'tileK', 'loadVector', 'ldsStage', 'ldsSwizzle',
+              'registerBudget', 'raster', 'finish']
+
+
+def sched_via_rule(ctx, s):
+    """Apply the rule sequence to the compute stage (the counterpart of
+    gpu_tensorcore_operator.py:362-414; one stage, since loads, MFMA and store are fused in the template)."""
+    stage_name = ctx.tensorize_info['stage_name']
+    for name in RULE_ORDER:
+        ctx.addSched(name, stage_name, s)

@@ -1,0 +1,112 @@
+"""Tune and time cases on MI355X:  python run.py -p rocm -c quick_start.json
+
+Same command line, JSON schema, output files (<out_name>/<case>/{schedule.py, constraints.py,
+records.txt, stat.txt}) and final ``PASS`` / ``Case ..., latency ... ms.`` lines as the reference's
+tests/quick_start/{dlboost,tensorcore}/run.py:19-110, with ``-p rocm`` selecting the MFMA operator
+set, the CDNA4 constraint set and the HIP measurer.  ``--check`` additionally verifies every
+measured kernel against a numpy host reference (Task.set_verify_func).
+"""
+import argparse
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.abspath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "..", ".."))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import heron_amd.ops.rocm as heron_rocm                              # noqa: E402
+import heron_amd.runner as HeronRunner                                # noqa: E402
+from heron_amd.config import configFromFile                           # noqa: E402
+from heron_amd.environment import Env                                 # noqa: E402
+from heron_amd import workloads                                       # noqa: E402
+
+
+def makeConfig(args):
+    config = configFromFile(args.config)
+    if args.platform == "rocm":
+        config.target_name = 'rocm'
+        config.codegen_type = 'GPU_MFMA'
+        config.get_op = heron_rocm.getOpFromName
+    return config
+
+
+def host_reference(op_name):
+    """numpy reference for --check: returns func(args) -> ([inputs], expected_output)."""
+    def gemm(params):
+        *shape, in_dtype, _ = params
+        if op_name == "gemm":
+            M, K, N = shape
+            if in_dtype == "float16":
+                A, B = workloads.gemm_f16_inputs(M, K, N)
+                return [A, B], (A.astype(np.float32) @ B.astype(np.float32).T)
+            A, B = workloads.gemm_u8s8_inputs(M, K, N)
+            return [A, B], (A.astype(np.int64) @ B.astype(np.int64).T)
+        b, M, K, N = shape
+        A, B = workloads.bmm_qk_inputs(b, M, K, N)
+        return [A, B], np.einsum("bik,bjk->bij", A.astype(np.float32), B.astype(np.float32))
+    return gemm
+
+
+def run(op_name, task_name, params, env, runner, check=False):
+    config = env.config
+    op = config.get_op(op_name)
+    task = env.createTask(task_name, op, params, config.target_name)
+    task.device_id = config.device_id
+    if check and op_name in ("gemm", "bmm"):
+        task.set_verify_func(host_reference(op_name), rtol=1e-2)
+    if config.tuned == "":
+        env.tune(task_name)
+        config.tuned = os.path.join(config.log_dir, 'records.txt')
+    s, args = task.apply_best(config.tuned)
+    print("Best instance:", s.describe())
+    latency = runner.time_instance(s, args, number=config.runner_number, repeat=config.runner_repeat,
+                                   min_repeat_ms=500) * 1e3
+    if latency > 0:
+        print("PASS")
+    return latency
+
+
+if __name__ == '__main__':
+    parser = argparse.ArgumentParser(description='Run cases in Heron.')
+    parser.add_argument("-p", "--platform", choices=['rocm'], type=str, default="rocm",
+                        help="Hardware platform: rocm (MI355X, MFMA templates).")
+    parser.add_argument("-c", "--config", type=str, required=True,
+                        help="Config file name: describes the param of test_cases")
+    parser.add_argument("-t", "--tuned", type=str, default="",
+                        help="records.txt of an earlier run: tuned parameters for direct use.")
+    parser.add_argument("-d", "--device_id", type=int, default=0, help="Device index for measurement")
+    parser.add_argument("-sid", "--start_id", type=int, default=0, help="Start case number in test cases")
+    parser.add_argument("-eid", "--end_id", type=int, default=int(1e4), help="End case number in test cases")
+    parser.add_argument("-v", "--verbose", action="store_true", help="Show some information if enabled.")
+    parser.add_argument("-m", "--max-trials", type=int, default=int(1e6), help="Max trials by command line")
+    parser.add_argument("--check", action="store_true", help="verify measured kernels against a host reference")
+    args = parser.parse_args()
+    print("Heron device ", args.device_id)
+
+    config = makeConfig(args)
+    config.max_trials = min(args.max_trials, config.max_trials)
+    config.device_id = args.device_id
+    config.tuned = args.tuned
+    config.verbose = args.verbose
+    runner = HeronRunner.LocalRunner(number=config.runner_number, repeat=config.runner_repeat, min_repeat_ms=0,
+                                     timeout=config.runner_timeout, device_id=args.device_id)
+    measure_option = HeronRunner.measure_option(
+        builder=HeronRunner.LocalBuilder(timeout=config.build_timeout),
+        runner=runner,
+    )
+    cases = []
+    case_keys = list(config.cases.keys())
+    for i in range(args.start_id, min(args.end_id + 1, len(case_keys))):
+        if i >= 1:
+            config.tuned = ''
+        op_name, case = config.cases[case_keys[i]]
+        print(case)
+        env = Env(measure_option, config)
+        latency = run(op_name, case_keys[i], case + [config.in_dtype, config.out_dtype], env, runner, args.check)
+        cases.append([case, latency])
+    for tup in cases:
+        print("Case %s, latency %f ms." % (str(tup[0]), tup[1]))
+    runner.close()
+    measure_option["builder"].close()

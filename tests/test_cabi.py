@@ -1,0 +1,65 @@
+"""The C ABI library loads and exports every symbol include/heron_rocm.h declares (no GPU needed)."""
+import ctypes
+import os
+import re
+
+from heron_amd import backend as B
+from heron_amd import instances
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "heron_rocm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hrn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_exported_and_bound():
+    names = declared_symbols()
+    assert len(names) >= 16
+    L = ctypes.CDLL(B.LIB_PATH)
+    for n in names:
+        assert hasattr(L, n), n
+    assert set(names) == set(B.SYMBOLS), set(names) ^ set(B.SYMBOLS)
+    assert b"gfx950" in B.lib().hrn_version()
+
+
+def test_struct_sizes_match_header_layout():
+    assert ctypes.sizeof(B.KernelDesc) == 16 * 4
+    assert ctypes.sizeof(B.KernelInfo) == 8 * 4
+    assert ctypes.sizeof(B.Problem) == 8 * 4 + 3 * 8 + 10 * 4 + 4 * 4
+    assert ctypes.sizeof(B.DevInfo) == 64 + 128 + 10 * 4 + 8
+
+
+def test_check_desc_mirrors_template_constraints():
+    ok = instances.D(instances.F16, instances.GEMM, 256, 256, 128, 2, 2, 32, 2, 2)
+    assert B.check_desc(ok) and B.lds_bytes(ok) == 131072
+    bad = [
+        instances.D(instances.F16, instances.GEMM, 256, 256, 128, 2, 2, 32, 3, 2),    # 192 KiB LDS
+        instances.D(instances.F16, instances.GEMM, 256, 256, 64, 2, 2, 16, 2, 0),     # one k-step per tile
+        instances.D(instances.F16, instances.GEMM, 96, 128, 128, 2, 2, 32, 2, 0),     # 96 rows / (2 waves x 32)
+        instances.D(instances.F16, instances.GEMM, 128, 128, 256, 2, 2, 16, 2, 2),    # swizzle period 32 > mfma 16
+        instances.D(instances.U8, instances.CONV, 128, 128, 128, 2, 2, 32, 2, 1),     # conv is fp16 only
+        instances.D(instances.F16, instances.GEMM, 512, 512, 64, 2, 2, 32, 2, 0),     # 1024 accumulators
+        instances.D(instances.F16, instances.GEMM, 128, 128, 128, 8, 4, 32, 2, 0),    # 32 waves
+    ]
+    for d in bad:
+        assert not B.check_desc(d), d
+        assert B.lib().hrn_last_error()
+
+
+def test_problem_helpers():
+    p = B.gemm_problem(3, 100, 200, 64)
+    assert (p.batch, p.m, p.n, p.k, p.lda, p.ldb, p.ldc, p.stride_c) == (3, 100, 200, 64, 64, 64, 200, 20000)
+    c = B.conv2d_problem(32, 56, 56, 64, 64, 3, 3, 1, 1, 1)
+    assert (c.m, c.n, c.k) == (32 * 56 * 56, 64, 576)
+    c = B.conv2d_problem(1, 15, 15, 8, 16, 3, 3, 2, 1, 1)
+    assert c.m == 8 * 8
+
+
+def test_compile_without_gpu_and_shipped_instances_present():
+    d = instances.BEST["small"]
+    path = B.compile_desc(d, 120.0)
+    assert path.endswith(".hsaco") and os.path.getsize(path) > 1000
+    assert os.path.exists(path[:-6] + ".info")

@@ -1,0 +1,130 @@
+"""Pins the CPU oracle (test infrastructure) independently of the HIP path.
+
+The reference holds no golden output for its operators, so each oracle function is pinned by
+checks that a plausible mistake (dropped term, wrong sign/index, transposed operand) fails:
+brute-force Python loops on tiny inputs, numpy int64 closed form, hardware ``vpdpbusd`` path vs the
+scalar loop, extreme-value closed forms, torch's CPU conv2d, identities and linearity.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from heron_amd import workloads
+
+
+def brute_gemm(A, B):
+    M, K = A.shape
+    N = B.shape[0]
+    C = [[0] * N for _ in range(M)]
+    for i in range(M):
+        for j in range(N):
+            s = 0
+            for k in range(K):
+                s += int(A[i, k]) * int(B[j, k])
+            C[i][j] = s
+    return np.array(C)
+
+
+def test_int_gemm_against_brute_force_and_numpy():
+    rng = np.random.default_rng(0)
+    A = rng.integers(0, 256, (5, 12), dtype=np.uint8)
+    B = rng.integers(-128, 128, (7, 12), dtype=np.int8)       # non-square: a transposed operand would not even fit
+    ref = brute_gemm(A, B)
+    assert np.array_equal(oracle.gemm_u8s8s32_scalar(A, B), ref)
+    assert np.array_equal(oracle.gemm_int64_numpy(A, B), ref)
+    assert np.array_equal(oracle.gemm_u8s8s32_dlboost(A, B), ref)     # scalar fallback (N % 32 != 0)
+
+
+def test_config1_gemm64_all_paths_agree():
+    A, B = workloads.gemm_u8s8_inputs(64, 64, 64, seed=0)
+    ref = oracle.gemm_int64_numpy(A, B)
+    assert np.array_equal(oracle.gemm_u8s8s32_scalar(A, B), ref)
+    C, path = oracle.gemm_u8s8s32_dlboost(A, B, return_path=True)
+    assert np.array_equal(C, ref)
+    if oracle.has_vnni():
+        assert path == 2          # the vpdpbusd micro-kernel really ran
+
+
+@pytest.mark.parametrize("M,K,N", [(13, 64, 32), (64, 128, 96), (200, 260, 160), (1, 4, 32)])
+def test_vnni_path_vs_scalar(M, K, N):
+    if not oracle.has_vnni():
+        pytest.skip("host has no AVX512-VNNI")
+    A, B = workloads.gemm_u8s8_inputs(M, K, N, seed=M)
+    C, path = oracle.gemm_u8s8s32_dlboost(A, B, return_path=True)
+    assert path == 2
+    assert np.array_equal(C, oracle.gemm_u8s8s32_scalar(A, B))
+    assert np.array_equal(oracle.PackedB(B).matmul(A), C)
+
+
+def test_int_extremes_closed_form():
+    """255 * -128 * K is the most negative sum; at K = 8192 it is -267386880 and fits int32."""
+    K = 8192
+    A = np.full((2, K), 255, np.uint8)
+    for bv, expect in ((-128, -267386880), (127, 255 * 127 * K)):
+        B = np.full((32, K), bv, np.int8)
+        for C in (oracle.gemm_u8s8s32_scalar(A, B), oracle.gemm_u8s8s32_dlboost(A, B)):
+            assert C.dtype == np.int32 and np.all(C == expect)
+    # unsigned A: 200 must count as +200, not as int8 -56
+    A = np.full((1, 4), 200, np.uint8)
+    B = np.ones((32, 4), np.int8)
+    assert np.all(oracle.gemm_u8s8s32_dlboost(A, B) == 800)
+
+
+def test_int_bmm_is_per_batch_gemm():
+    rng = np.random.default_rng(3)
+    A = rng.integers(0, 256, (3, 6, 8), dtype=np.uint8)
+    B = rng.integers(-128, 128, (3, 5, 8), dtype=np.int8)
+    C = oracle.bmm_u8s8s32_scalar(A, B)
+    for b in range(3):
+        assert np.array_equal(C[b], brute_gemm(A[b], B[b]))
+
+
+def test_f32_gemm_and_bmm_against_float64():
+    A, B = workloads.gemm_f16_inputs(33, 72, 17, seed=2)
+    ref = oracle.gemm_f64_numpy(A, B)
+    got = oracle.gemm_f32(A, B)
+    assert got.shape == (33, 17)
+    assert np.abs(got - ref).max() <= 1e-6 * np.abs(ref).max()
+    Q, Kt = workloads.bmm_qk_inputs(3, 10, 16, 12)
+    assert np.abs(oracle.bmm_f32(Q, Kt) - oracle.bmm_f64_numpy(Q, Kt)).max() < 1e-5
+    # identity B returns A
+    eye = np.eye(72, dtype=np.float16)
+    assert np.array_equal(oracle.gemm_f32(A, eye), A.astype(np.float32))
+
+
+CONV = [(2, 9, 11, 8, 6, 3, 3, 1, 1, 1), (1, 8, 8, 4, 5, 1, 1, 1, 0, 1), (1, 13, 12, 3, 4, 3, 3, 2, 1, 1),
+        (2, 10, 10, 2, 3, 3, 3, 1, 2, 2), (1, 7, 9, 4, 2, 5, 3, 1, 0, 1), (1, 12, 12, 2, 2, 3, 3, 3, 2, 2)]
+
+
+@pytest.mark.parametrize("case", CONV)
+def test_conv_against_torch_library_routine(case):
+    N, H, W, CI, CO, KH, KW, s, p, d = case
+    X, Wt = workloads.conv2d_inputs(N, H, W, CI, CO, KH, KW, seed=sum(case))
+    got = oracle.conv2d_nhwc_f32(X, Wt, s, p, d)
+    x = torch.from_numpy(X.astype(np.float64)).permute(0, 3, 1, 2)            # NHWC -> NCHW
+    w = torch.from_numpy(Wt.astype(np.float64)).permute(0, 3, 1, 2)           # KRSC -> KCRS
+    ref = torch.nn.functional.conv2d(x, w, stride=s, padding=p, dilation=d).permute(0, 2, 3, 1).numpy()
+    assert got.shape == ref.shape                                              # output-size formula
+    assert got.shape[1:3] == workloads.conv_out_hw(H, W, KH, KW, s, p, d)
+    assert np.abs(got - ref).max() <= 1e-5 * (np.abs(ref).max() + 1)
+
+
+def test_conv_1x1_reduces_to_gemm():
+    X, Wt = workloads.conv2d_inputs(2, 5, 6, 8, 7, 1, 1, seed=9)
+    got = oracle.conv2d_nhwc_f32(X, Wt)
+    ref = oracle.gemm_f32(X.reshape(-1, 8), Wt.reshape(7, 8)).reshape(2, 5, 6, 7)
+    assert np.array_equal(got, ref)
+
+
+def test_workload_generators_are_seeded_and_shaped():
+    A1, B1 = workloads.gemm_u8s8_inputs(64, 64, 64, seed=0)
+    A2, B2 = workloads.gemm_u8s8_inputs(64, 64, 64, seed=0)
+    assert np.array_equal(A1, A2) and np.array_equal(B1, B2)
+    assert A1.dtype == np.uint8 and B1.dtype == np.int8 and A1.max() > 200 and B1.min() < -100
+    P, Vt = workloads.bmm_pv_inputs(2, 8, 16, 4)
+    assert np.abs(P.astype(np.float32).sum(-1) - 1).max() < 1e-2
+    X, _ = workloads.conv2d_inputs(1, 8, 8, 8, 8, 3, 3)
+    assert 0.3 < (X == 0).mean() < 0.7
+    assert workloads.gemm_work(8192, 8192, 8192, 1, 4) == (2 * 8192 ** 3, 402653184)
+    assert workloads.conv_work(32, 56, 56, 64, 64, 3, 3, 1, 1, 1) == (7398752256, 25763840)

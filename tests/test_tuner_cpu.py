@@ -1,0 +1,206 @@
+"""Host logic of the tuning stack on CPU: template sampling, CGA loop, records, failure handling.
+
+The GPU is replaced by a synthetic measurer with the builder/runner interface (set_task,
+get_build_kwargs, build, run): latency comes from a closed-form model of the template parameters,
+so the search has something to optimise and the tests stay deterministic enough.
+"""
+import copy
+import json
+import math
+import os
+import time
+
+import numpy as np
+import pytest
+
+from heron_amd import backend as B
+from heron_amd.config import Config
+from heron_amd.environment import Env
+from heron_amd.multi import Job
+from heron_amd.ops.rocm import getOpFromName
+from heron_amd.runner import MeasureErrorNo, MeasureResult, Runner, measure_option
+from heron_amd.runner.measure import BuildResult
+from heron_amd.task import Task
+
+
+class FakeBuilder:
+    n_parallel = 2
+
+    def set_task(self, task, build_kwargs=None):
+        self.task = task
+
+    def build(self, inputs):
+        out = []
+        for inp in inputs:
+            s, args = inp.task.instantiate(inp.config)
+            err = None if B.check_desc(s.to_desc()) else (MeasureErrorNo.INSTANTIATION_ERROR, "bad desc")
+            out.append(BuildResult(s.to_desc().as_tuple(), dict(s.params), None, err, 0.0))
+        return out
+
+
+class FakeRunner:
+    """Latency model: bigger tiles and 2 waves/SIMD are faster; one instance family 'fails to launch'."""
+
+    def __init__(self):
+        self.calls = 0
+
+    def set_task(self, task):
+        return None
+
+    def get_build_kwargs(self):
+        return {'check_gpu': {'lds_bytes_per_wg': 163840, 'max_threads_per_wg': 1024, 'wave_size': 64,
+                              'regs_per_simd_lane': 512, 'simd_per_cu': 4, 'cu_count': 256}}
+
+    def run(self, inputs, builds):
+        res = []
+        for inp, br in zip(inputs, builds):
+            self.calls += 1
+            if br.error is not None:
+                res.append(MeasureResult((RuntimeError(br.error[1]),), br.error[0], 0.0, time.time()))
+                continue
+            p = br.problem
+            if p['bm'] == 16 and p['bn'] == 16:
+                res.append(MeasureResult((RuntimeError("launch failed"),), MeasureErrorNo.RUNTIME_DEVICE, 0.0, time.time()))
+                continue
+            cost = 1e-3 * (1 + 64.0 / p['bm'] + 64.0 / p['bn'] + 0.1 * abs(p['stages'] - 3) + (0.3 if p['mfma'] == 16 else 0))
+            res.append(MeasureResult(cost, 0, 0.01, time.time()))
+        return res
+
+
+def make_env(tmp_path, method="CGA", trials=48, case=("gemm", [1024, 1024, 1024]), dtype="float16"):
+    cfg = Config()
+    cfg.codegen_type, cfg.target_name, cfg.get_op = 'GPU_MFMA', 'rocm', getOpFromName
+    cfg.out_name = str(tmp_path / "OPS")
+    cfg.opt_method, cfg.max_trials = method, trials
+    cfg.measure_time_per_round, cfg.pop_num, cfg.select_num, cfg.iter_walks = 16, 24, 12, 2
+    cfg.parallel_num, cfg.history_topk = 2, 8
+    cfg.in_dtype, cfg.out_dtype = dtype, dtype
+    env = Env(measure_option(FakeBuilder(), FakeRunner()), cfg)
+    op, shape = case
+    env.createTask("T1", cfg.get_op(op), shape + [cfg.in_dtype, cfg.out_dtype], cfg.target_name)
+    return env
+
+
+@pytest.mark.parametrize("op,shape,dtype", [("gemm", [8192, 8192, 8192], "float16"), ("gemm", [64, 64, 64], "int8"),
+                                            ("bmm", [192, 512, 64, 512], "float16"),
+                                            ("c2d", [32, 56, 56, 64, 64, 3, 3, 1, 1, 1], "float16")])
+def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
+    """The Python constraint set and hrn_check_desc describe the same template space."""
+    cfg = Config()
+    cfg.codegen_type = 'GPU_MFMA'
+    t = Task("t", getOpFromName(op), shape + [dtype, dtype], "rocm")
+    t.config = cfg
+    t.make_stage_schedules()
+    assert len(t.knob_manager.knob_names) == 10 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
+    seen = set()
+    for _ in range(40):
+        km = copy.deepcopy(t.knob_manager)
+        valid, point = km.randSample({})
+        s, args = t.instantiate(km)
+        d = s.to_desc()
+        assert valid and B.check_desc(d), (d, B.lib().hrn_last_error())
+        g = s.info['gemm_view']
+        assert g['M'] <= math.ceil(g['M'] / d.bm) * d.bm and (16 * math.ceil(g['M'] / 16)) % d.bm == 0
+        assert B.lds_bytes(d) == km.solved_knob_vals_phenotype[[k for k in km.solver.vals if k.endswith("VA:lds_bytes")][0]]
+        assert [a.name for a in args][-1] == s.info['stage_name']
+        seen.add(d.as_tuple())
+    assert len(seen) > 20
+    # the hand-picked 256x256 instance is inside the space (fp16/int8 GEMM)
+    if op == "gemm" and shape[0] == 8192:
+        km = copy.deepcopy(t.knob_manager)
+        P = lambda n: "P#ST:dense,AX:None,PA:%s" % n
+        _, ok = km.validate({P('mfma'): 32, P('wave_m'): 2, P('wave_n'): 2, P('tile_m'): 4, P('tile_n'): 4,
+                             P('block_k_bytes'): 128, P('lds_stages'): 2, P('lds_swizzle'): 2})
+        assert ok
+        _, ok = km.validate({P('mfma'): 32, P('wave_m'): 2, P('wave_n'): 2, P('tile_m'): 4, P('tile_n'): 4,
+                             P('block_k_bytes'): 128, P('lds_stages'): 3})
+        assert not ok                                            # 192 KiB of LDS
+
+
+def test_cga_tuning_loop_writes_reference_format(tmp_path):
+    env = make_env(tmp_path)
+    np.random.seed(0)
+    env.tune("T1")
+    log = env.config.log_dir
+    for f in ("schedule.py", "constraints.py", "records.txt", "stat.txt"):
+        assert os.path.exists(os.path.join(log, f)), f
+    rows = [json.loads(l) for l in open(os.path.join(log, "records.txt"))]
+    assert 30 <= len(rows) <= 48
+    for r in rows:
+        assert set(r) == {"code", "perf", "latency", "time", "param"}
+        assert r["perf"] == 0.0 or abs(r["latency"] - math.exp(-r["perf"])) < 1e-12
+        assert len(r["code"].split("_")) - 1 == len(r["param"])
+    stat = [l.strip().split(",") for l in open(os.path.join(log, "stat.txt"))]
+    assert len(stat) == math.ceil(48 / 16) + 1 and all(len(x) == 6 for x in stat)
+    # the search found a good point of the synthetic model (optimum 1.5 ms at 256x256, 3 stages)
+    best = max(r["perf"] for r in rows)
+    assert math.exp(-best) < 2.2e-3
+    # failed launches were recorded with perf 0 and kept out of the training data
+    assert all(y != 0 for y in env.perf_buffer.data_y)
+    # apply_best re-instantiates the best record
+    t2 = make_env(tmp_path / "again").task
+    s, args = t2.apply_best(os.path.join(log, "records.txt"))
+    best_row = max(rows, key=lambda r: r["perf"])
+    assert s.params['bm'] == best_row["param"]["V#ST:dense,AX:None,VA:block_m"]
+    assert "mfma" in t2.getStmt(t2.knob_manager)
+    # constraints.py is re-loadable and equals the live constraint system
+    from heron_amd.schedule.constraints import Solver
+    again = Solver.from_dump(open(os.path.join(log, "constraints.py")).read())
+    assert len(again.vals) == len(env.task.knob_manager.solver.vals)
+    from heron_amd.schedule.constraints.primitives import removedot
+    assert again.SATScore({removedot(k): v for k, v in best_row["param"].items()}) == 0
+
+
+def test_crand_tuner_and_last_round_quirk(tmp_path):
+    """max_trials a multiple of the round size: the final round measures nothing (tuner.py:50-58 of the reference)."""
+    env = make_env(tmp_path, method="CRAND", trials=32)
+    env.tune("T1")
+    rows = [json.loads(l) for l in open(os.path.join(env.config.log_dir, "records.txt"))]
+    assert len(rows) <= 32
+    stat = open(os.path.join(env.config.log_dir, "stat.txt")).read().strip().splitlines()
+    assert len(stat) == 3
+
+
+def test_results2tup_and_error_mapping():
+    r = Runner(None)
+    res = r.results2tup([MeasureResult(2e-6, 0, 0, 0), MeasureResult((RuntimeError("x"),), MeasureErrorNo.RUN_TIMEOUT, 0, 0),
+                         MeasureResult([1e-3, 3e-3], 0, 0, 0), MeasureResult(1e-3, MeasureErrorNo.VERIFY_FAILED, 0, 0)])
+    assert res[0] == (0, math.log(1 / 2e-6)) and res[1] == (MeasureErrorNo.RUN_TIMEOUT, 0.0)
+    assert abs(res[2][1] - math.log(1 / 2e-3)) < 1e-12 and res[3] == (100, 0.0)
+
+
+def _sleepy(seconds):
+    time.sleep(seconds)
+    return [1]
+
+
+def test_job_timeout_kills_the_child():
+    job = Job(_sleepy, (30,), timeout=0.5)
+    t0 = time.time()
+    job.start(job.attach_info)
+    assert job.get() == 0 and time.time() - t0 < 10
+    job = Job(_sleepy, (0,), timeout=10)
+    job.start(job.attach_info)
+    assert job.get() == [1]
+
+
+def test_cost_model_learns_and_ranks():
+    from heron_amd.model import XGBoostCostModel
+
+    class T:
+        target = "rocm"
+
+    class S:
+        def __init__(self, p):
+            self.point = p
+    cfg = Config()
+    m = XGBoostCostModel(T(), cfg)
+    rng = np.random.default_rng(0)
+    X = rng.integers(0, 8, (200, 6))
+    y = 10 + X[:, 0] * 0.5 - X[:, 3] * 0.3
+    assert np.all(m.predict([S(list(x)) for x in X[:5]]) == 1)           # untrained -> ones
+    m.fit(X, y)
+    pred = m.predict([S(list(x)) for x in X])
+    assert np.corrcoef(pred, y)[0, 1] > 0.95
+    score = m.bst.get_score()
+    assert max(score, key=score.get) in ("f0", "f3")
