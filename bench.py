@@ -30,7 +30,9 @@ def make_workloads(torch, workloads, instances):
 
     W = {}
 
-    def add_gemm(name, key, M, K, N, f16, batch=1, gen=None, group_m=8):
+    def add_gemm(name, key, M, K, N, f16, batch=1, gen=None):
+        group_m = instances.BEST_GROUP_M.get(key, 8)
+
         def build():
             if gen is not None:
                 A, Bm = gen()

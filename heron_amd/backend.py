@@ -49,9 +49,11 @@ class KernelDesc(ctypes.Structure):
     _fields_ = [("dtype", ctypes.c_int32), ("op", ctypes.c_int32), ("bm", ctypes.c_int32), ("bn", ctypes.c_int32),
                 ("bkb", ctypes.c_int32), ("wm", ctypes.c_int32), ("wn", ctypes.c_int32), ("mfma", ctypes.c_int32),
                 ("stages", ctypes.c_int32), ("swizzle", ctypes.c_int32), ("epilogue", ctypes.c_int32),
-                ("waves_per_eu", ctypes.c_int32), ("reserved", ctypes.c_int32 * 4)]
+                ("waves_per_eu", ctypes.c_int32), ("l2_prefetch", ctypes.c_int32), ("ablate", ctypes.c_int32),
+                ("reserved", ctypes.c_int32 * 2)]
 
-    KEYS = ("dtype", "op", "bm", "bn", "bkb", "wm", "wn", "mfma", "stages", "swizzle", "epilogue", "waves_per_eu")
+    KEYS = ("dtype", "op", "bm", "bn", "bkb", "wm", "wn", "mfma", "stages", "swizzle", "epilogue", "waves_per_eu",
+            "l2_prefetch", "ablate")
 
     def as_tuple(self):
         return tuple(int(getattr(self, k)) for k in self.KEYS)
@@ -81,8 +83,9 @@ class Problem(ctypes.Structure):
 
 
 def make_desc(dtype, op=HRN_OP_GEMM, bm=128, bn=128, bkb=128, wm=2, wn=2, mfma=32, stages=2, swizzle=1,
-              epilogue=0, waves_per_eu=0):
+              epilogue=0, waves_per_eu=0, l2_prefetch=0, ablate=0):
     d = KernelDesc()
+    d.l2_prefetch, d.ablate = l2_prefetch, ablate
     d.dtype, d.op, d.bm, d.bn, d.bkb, d.wm, d.wn = dtype, op, bm, bn, bkb, wm, wn
     d.mfma, d.stages, d.swizzle, d.epilogue, d.waves_per_eu = mfma, stages, swizzle, epilogue, waves_per_eu
     return d
@@ -126,6 +129,8 @@ SYMBOLS = {
     "hrn_time": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _i, _d, ctypes.POINTER(_d), _vp]),
     "hrn_problem_gemm": (None, [ctypes.POINTER(Problem), _i, _i, _i, _i]),
     "hrn_problem_conv2d": (None, [ctypes.POINTER(Problem)] + [_i] * 10),
+    "hrn_probe_mfma": (_i, [_i, _i, _i, ctypes.POINTER(_d), _vp]),
+    "hrn_probe_copy": (_i, [_vp, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_last_error": (ctypes.c_char_p, []),
     "hrn_version": (ctypes.c_char_p, []),
 }
@@ -190,6 +195,20 @@ def conv2d_problem(n, h, w, ci, co, kh, kw, stride, pad, dil, group_m=8):
     lib().hrn_problem_conv2d(ctypes.byref(p), n, h, w, ci, co, kh, kw, stride, pad, dil)
     p.group_m = group_m
     return p
+
+
+def probe_mfma(dtype, mfma=32, random_operands=True, stream=0):
+    """Dense T(FL)OP/s of a register-resident MFMA loop on all CUs (measured roofline denominator)."""
+    out = _d()
+    _check(lib().hrn_probe_mfma(dtype, mfma, 1 if random_operands else 0, ctypes.byref(out), stream))
+    return out.value
+
+
+def probe_copy(src_ptr, dst_ptr, nbytes, repeat=10, stream=0):
+    """GB/s (read + write) of a plain 16-byte-per-lane copy kernel over caller-owned device memory."""
+    out = _d()
+    _check(lib().hrn_probe_copy(src_ptr, dst_ptr, nbytes, repeat, ctypes.byref(out), stream))
+    return out.value
 
 
 class Module:

@@ -23,6 +23,7 @@
 #include <sstream>
 #include <string>
 #include <thread>
+#include <type_traits>
 #include <vector>
 
 #define HRN_KARGS_DEFINED
@@ -114,10 +115,11 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (d->mfma != 32 && d->mfma != 16) return fail(HRN_E_BADPARAM, "mfma %d not in {16,32}", d->mfma);
     if (d->wm < 1 || d->wn < 1 || d->wm * d->wn > 16) return fail(HRN_E_BADPARAM, "wave grid %dx%d", d->wm, d->wn);
     if (d->bm < 16 || d->bn < 16 || d->bm > 512 || d->bn > 512) return fail(HRN_E_BADPARAM, "tile %dx%d", d->bm, d->bn);
-    if (d->stages < 2 || d->stages > 4) return fail(HRN_E_BADPARAM, "stages %d not in 2..4", d->stages);
+    if (d->stages < 2 || d->stages > 5) return fail(HRN_E_BADPARAM, "stages %d not in 2..5", d->stages);
     if (d->swizzle < 0 || d->swizzle > 3) return fail(HRN_E_BADPARAM, "swizzle %d", d->swizzle);
     if (d->epilogue < 0 || d->epilogue > 1) return fail(HRN_E_BADPARAM, "epilogue %d", d->epilogue);
     if (d->waves_per_eu < 0 || d->waves_per_eu > 8) return fail(HRN_E_BADPARAM, "waves_per_eu %d", d->waves_per_eu);
+    if (d->l2_prefetch < 0 || d->l2_prefetch > 8) return fail(HRN_E_BADPARAM, "l2_prefetch %d not in 0..8", d->l2_prefetch);
     Derived r;
     r.es = d->dtype == HRN_DT_F16 ? 2 : 1;
     r.nw = d->wm * d->wn;
@@ -137,13 +139,21 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     r.tm = d->bm / d->wm / d->mfma;
     r.tn = d->bn / d->wn / d->mfma;
     r.stage_bytes = (d->bm + d->bn) * d->bkb;
-    r.lds = d->stages * r.stage_bytes;
+    r.lds = d->stages * r.stage_bytes + (d->l2_prefetch ? r.nw * 256 : 0);
     if (r.lds > 163840) return fail(HRN_E_BADPARAM, "LDS %d > 163840", r.lds);
     if (d->swizzle && (r.cpr << (d->swizzle - 1)) > d->mfma)
         return fail(HRN_E_BADPARAM, "swizzle %d period %d exceeds mfma %d", d->swizzle, r.cpr << (d->swizzle - 1), d->mfma);
     if (d->op == HRN_OP_CONV2D && d->swizzle && (r.nw * r.rpi) % (r.cpr << (d->swizzle - 1)))
         return fail(HRN_E_BADPARAM, "conv: swizzle period must divide rows per load round");
-    if ((d->stages - 1) * r.lpt > 63) return fail(HRN_E_BADPARAM, "too many loads in flight (%d)", (d->stages - 1) * r.lpt);
+    {
+        // every tile fetch may be preceded by the prefetch touches of a later tile
+        const int lines = (d->bm + d->bn) * ((d->bkb + 127) / 128);
+        if (d->l2_prefetch && d->op != HRN_OP_GEMM) return fail(HRN_E_BADPARAM, "l2_prefetch is for GEMM only");
+        if (d->l2_prefetch && (d->bm * ((d->bkb + 127) / 128)) % 64) return fail(HRN_E_BADPARAM, "l2_prefetch needs bm*lines_per_row %% 64 == 0");
+        const int pf = d->l2_prefetch ? (lines + r.nw * 64 - 1) / (r.nw * 64) : 0;
+        if ((d->stages - 1) * (r.lpt + pf) > 63)
+            return fail(HRN_E_BADPARAM, "too many loads in flight (%d)", (d->stages - 1) * (r.lpt + pf));
+    }
     const int acc = r.tm * r.tn * (d->mfma == 32 ? 16 : 4);
     if (acc > 256) return fail(HRN_E_BADPARAM, "accumulators %d > 256 registers per lane", acc);
     if (d->dtype == HRN_DT_U8S8 && d->bn * 4 > r.lds) return fail(HRN_E_BADPARAM, "LDS too small for the column sums");
@@ -153,8 +163,8 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
 
 std::string desc_key(const hrn_kernel_desc* d, uint64_t srch) {
     char b[256];
-    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_%08x", d->dtype, d->op, d->bm, d->bn,
-             d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu,
+    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_a%d_f%d_%08x", d->dtype, d->op, d->bm, d->bn,
+             d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu, d->ablate, d->l2_prefetch,
              (unsigned)(srch ^ (srch >> 32)));
     return b;
 }
@@ -230,6 +240,8 @@ int compile_desc(const hrn_kernel_desc* d, double timeout_s, std::string* out_pa
     def("HRN_BKB", d->bkb); def("HRN_WM", d->wm); def("HRN_WN", d->wn); def("HRN_MFMA", d->mfma);
     def("HRN_STAGES", d->stages); def("HRN_SWZ", d->swizzle); def("HRN_EPI", d->epilogue);
     def("HRN_WPE", d->waves_per_eu);
+    def("HRN_ABLATE", d->ablate);   // diagnostic switches of the template, 0 in normal use
+    def("HRN_PF", d->l2_prefetch);
     args.push_back(src);
     args.push_back("-o");
     args.push_back(co_tmp);
@@ -325,9 +337,147 @@ int launch(const hrn_module* mod, const hrn_problem* p, const void* A, const voi
     return HRN_OK;
 }
 
+// ---- roofline probes -----------------------------------------------------------------------
+typedef int pv4i __attribute__((ext_vector_type(4)));
+typedef _Float16 pv8h __attribute__((ext_vector_type(8)));
+typedef float pv16f __attribute__((ext_vector_type(16)));
+typedef float pv4f __attribute__((ext_vector_type(4)));
+typedef int pv16i __attribute__((ext_vector_type(16)));
+
+// KIND 0: f16 32x32x16, 1: f16 16x16x32, 2: i8 32x32x32, 3: i8 16x16x64; 4 independent accumulators
+template <int KIND>
+__global__ void __launch_bounds__(256) probe_mfma_kernel(float* sink, int iters, int random_operands) {
+    pv4i a = {(int)threadIdx.x, 1, 2, 3}, b = {4, 5, 6, (int)blockIdx.x};
+    if (random_operands) {
+        // operands with the bit statistics of real data: fp16 values of magnitude ~2^-3..2^0 with random
+        // sign and mantissa, or uniformly random bytes (data-dependent switching power is part of the roofline)
+        uint32_t h = (threadIdx.x * 2654435761u) ^ (blockIdx.x * 40503u + 0x9e3779b9u);
+        for (int r = 0; r < 4; ++r) {
+            uint32_t w[2];
+            for (int q = 0; q < 2; ++q) {
+                h = h * 1664525u + 1013904223u;
+                uint32_t x = h ^ (h >> 15);
+                if (KIND < 2) {   // two halves: sign(1) exp in {12,13,14,15} mantissa(10)
+                    uint32_t lo = (x & 0x83ffu) | ((12u + ((x >> 10) & 3u)) << 10);
+                    uint32_t hi = ((x >> 16) & 0x83ffu) | ((12u + ((x >> 26) & 3u)) << 10);
+                    w[q] = lo | (hi << 16);
+                } else {
+                    w[q] = x;
+                }
+            }
+            a[r] = (int)w[0];
+            b[r] = (int)w[1];
+        }
+    }
+    if constexpr (KIND == 0 || KIND == 2) {
+        using acc_t = typename std::conditional<KIND == 0, pv16f, pv16i>::type;
+        acc_t c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
+        for (int i = 0; i < iters; ++i) {
+            if constexpr (KIND == 0) {
+                c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pv8h, a), __builtin_bit_cast(pv8h, b), c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pv8h, a), __builtin_bit_cast(pv8h, b), c1, 0, 0, 0);
+                c2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pv8h, a), __builtin_bit_cast(pv8h, b), c2, 0, 0, 0);
+                c3 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pv8h, a), __builtin_bit_cast(pv8h, b), c3, 0, 0, 0);
+            } else {
+                c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c1, 0, 0, 0);
+                c2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c2, 0, 0, 0);
+                c3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c3, 0, 0, 0);
+            }
+        }
+        float s = 0;
+        for (int r = 0; r < 16; ++r) s += (float)(c0[r] + c1[r] + c2[r] + c3[r]);
+        if (s == 123.456f) sink[0] = s;
+    } else {
+        using acc_t = typename std::conditional<KIND == 1, pv4f, pv4i>::type;
+        acc_t c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
+        for (int i = 0; i < iters; ++i) {
+            if constexpr (KIND == 1) {
+                c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pv8h, a), __builtin_bit_cast(pv8h, b), c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pv8h, a), __builtin_bit_cast(pv8h, b), c1, 0, 0, 0);
+                c2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pv8h, a), __builtin_bit_cast(pv8h, b), c2, 0, 0, 0);
+                c3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pv8h, a), __builtin_bit_cast(pv8h, b), c3, 0, 0, 0);
+            } else {
+                c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c1, 0, 0, 0);
+                c2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c2, 0, 0, 0);
+                c3 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c3, 0, 0, 0);
+            }
+        }
+        float s = 0;
+        for (int r = 0; r < 4; ++r) s += (float)(c0[r] + c1[r] + c2[r] + c3[r]);
+        if (s == 123.456f) sink[0] = s;
+    }
+}
+
+__global__ void __launch_bounds__(256) probe_copy_kernel(const pv4i* __restrict__ src, pv4i* __restrict__ dst, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
 }  // namespace
 
 extern "C" {
+
+int hrn_probe_mfma(int dtype, int mfma, int random_operands, double* tops_out, void* stream) {
+    if (!tops_out || (mfma != 32 && mfma != 16) || (dtype != HRN_DT_F16 && dtype != HRN_DT_U8S8))
+        return fail(HRN_E_BADPARAM, "probe arguments");
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t pr;
+    HIP_TRY(hipGetDeviceProperties(&pr, dev));
+    hipStream_t st = (hipStream_t)stream;
+    const int iters = 20000, grid = pr.multiProcessorCount * 2;   // 2 workgroups x 4 waves per CU: 2 waves per SIMD
+    const int kind = (dtype == HRN_DT_F16 ? 0 : 2) + (mfma == 32 ? 0 : 1);
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    float ms = 0;
+    for (int rep = 0; rep < 2; ++rep) {   // first pass warms up
+        (void)hipEventRecord(e0, st);
+        switch (kind) {
+            case 0: probe_mfma_kernel<0><<<grid, 256, 0, st>>>(nullptr, iters, random_operands); break;
+            case 1: probe_mfma_kernel<1><<<grid, 256, 0, st>>>(nullptr, iters, random_operands); break;
+            case 2: probe_mfma_kernel<2><<<grid, 256, 0, st>>>(nullptr, iters, random_operands); break;
+            default: probe_mfma_kernel<3><<<grid, 256, 0, st>>>(nullptr, iters, random_operands); break;
+        }
+        (void)hipEventRecord(e1, st);
+        hipError_t e = hipEventSynchronize(e1);
+        if (e != hipSuccess) { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); return fail(HRN_E_LAUNCH, "probe: %s", hipGetErrorString(e)); }
+        (void)hipEventElapsedTime(&ms, e0, e1);
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    const double ops_per_mfma = (dtype == HRN_DT_F16) ? 32768.0 : 65536.0;   // 2*m*n*k for either shape
+    const double total = ops_per_mfma * (mfma == 32 ? 1.0 : 0.5) * 4.0 * iters * 4.0 * grid;  // 4 accumulators, 4 waves
+    *tops_out = total / (ms * 1e-3) / 1e12;
+    return HRN_OK;
+}
+
+int hrn_probe_copy(const void* src, void* dst, size_t bytes, int repeat, double* gbs_out, void* stream) {
+    if (!src || !dst || !gbs_out || bytes < 16 || bytes % 16 || repeat < 1) return fail(HRN_E_BADPARAM, "probe arguments");
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t pr;
+    HIP_TRY(hipGetDeviceProperties(&pr, dev));
+    hipStream_t st = (hipStream_t)stream;
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    const int grid = pr.multiProcessorCount * 16;
+    probe_copy_kernel<<<grid, 256, 0, st>>>((const pv4i*)src, (pv4i*)dst, bytes / 16);
+    (void)hipEventRecord(e0, st);
+    for (int i = 0; i < repeat; ++i) probe_copy_kernel<<<grid, 256, 0, st>>>((const pv4i*)src, (pv4i*)dst, bytes / 16);
+    (void)hipEventRecord(e1, st);
+    hipError_t e = hipEventSynchronize(e1);
+    float ms = 0;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (e != hipSuccess) return fail(HRN_E_LAUNCH, "probe: %s", hipGetErrorString(e));
+    *gbs_out = 2.0 * bytes * repeat / (ms * 1e-3) / 1e9;
+    return HRN_OK;
+}
 
 const char* hrn_last_error(void) { return g_err.c_str(); }
 const char* hrn_version(void) { return "heron-rocm 0.1 (gfx950)"; }

@@ -51,6 +51,20 @@ constexpr int OP = HRN_OP;
 constexpr int BM = HRN_BM, BN = HRN_BN, BKB = HRN_BKB;
 constexpr int WM = HRN_WM, WN = HRN_WN, MT = HRN_MFMA, NS = HRN_STAGES, SWZ = HRN_SWZ;
 constexpr int EPI = HRN_EPI;
+// Diagnostic switches for bottleneck analysis (results are WRONG when non-zero; 0 in every shipped
+// instance): 1 skip LDS fragment reads after the first tile, 2 skip global->LDS loads after the
+// prologue, 4 drop the per-tile barrier, 8 skip the MFMAs.
+#ifndef HRN_ABLATE
+#define HRN_ABLATE 0
+#endif
+constexpr int ABL = HRN_ABLATE;
+// L2 prefetch: with HRN_PF = d > 0 every tile fetch is preceded by one 4-byte load per 128-byte line of the
+// k-tile d tiles further on.  The data is discarded; the point is that the line is in L2 (not HBM) when the
+// real fetch arrives, because a tile is only usable when its slowest load has landed.
+#ifndef HRN_PF
+#define HRN_PF 0
+#endif
+constexpr int PF = HRN_PF;
 constexpr int ES = (DT == 0) ? 2 : 1;       // input element bytes
 constexpr int OES = (DT == 0) ? 2 : 4;      // output element bytes
 constexpr int NW = WM * WN, NT = NW * 64;
@@ -58,7 +72,9 @@ constexpr int CPR = BKB / 16;               // 16-byte chunks per tile row
 constexpr int RPI = 64 / CPR;               // tile rows one wave load instruction covers
 constexpr int A_LPW = (BM / RPI) / NW;      // load instructions per wave per tile
 constexpr int B_LPW = (BN / RPI) / NW;
-constexpr int LPT = A_LPW + B_LPW;
+constexpr int LPR = (BKB + 127) / 128;                         // 128-byte lines per tile row
+constexpr int PF_N = PF ? ((BM + BN) * LPR + NW * 64 - 1) / (NW * 64) : 0;   // prefetch touches per lane per tile
+constexpr int LPT = A_LPW + B_LPW + PF_N;                       // vector memory ops per lane per tile
 constexpr int KSB = (MT == 32) ? 32 : 64;   // bytes of K one MFMA consumes
 constexpr int KS = BKB / KSB;               // MFMA k-steps per tile
 constexpr int CPS = KSB / 16;               // chunks per k-step (= 64 / MT)
@@ -72,9 +88,12 @@ static_assert(BKB == 64 || BKB == 128 || BKB == 256, "BKB");
 static_assert(MT == 32 || MT == 16, "MFMA");
 static_assert(KS >= 2 && (KS % 2) == 0, "need an even number of k-steps per tile");
 static_assert((BM / RPI) % NW == 0 && (BN / RPI) % NW == 0 && A_LPW >= 1 && B_LPW >= 1, "loads per wave");
+static_assert(OP == 0 || PF == 0, "L2 prefetch is implemented for the GEMM address pattern only");
+static_assert(PF == 0 || (BM * ((BKB + 127) / 128)) % 64 == 0, "L2 prefetch: A lines must fill whole waves");
 static_assert(BM % (WM * MT) == 0 && BN % (WN * MT) == 0, "wave tile");
-static_assert(NS >= 2 && NS <= 4, "stages");
-static_assert(NS * STAGE_BYTES <= 163840, "LDS");
+static_assert(NS >= 2 && NS <= 5, "stages");
+constexpr int PF_SCRATCH = PF ? NW * 256 : 0;                   // LDS corner the prefetch touches land in
+static_assert(NS * STAGE_BYTES + PF_SCRATCH <= 163840, "LDS");
 static_assert(SWZ == 0 || (CPR << (SWZ - 1)) <= MT, "swizzle period must fit in one MFMA tile");
 static_assert((NS - 1) * LPT <= 63, "vmcnt range");
 static_assert(NT <= 1024, "threads");
@@ -102,6 +121,13 @@ __device__ __forceinline__ void wait_and_barrier() {
     constexpr int vm = VM > 63 ? 63 : VM;
     constexpr int imm = (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((LGKM & 15) << 8);
     asm volatile("s_waitcnt %0\n\ts_barrier" ::"n"(imm) : "memory");
+}
+
+template <int VM, int LGKM>
+__device__ __forceinline__ void wait_only() {
+    constexpr int vm = VM > 63 ? 63 : VM;
+    constexpr int imm = (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((LGKM & 15) << 8);
+    asm volatile("s_waitcnt %0" ::"n"(imm) : "memory");
 }
 
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
@@ -149,7 +175,7 @@ extern "C" __global__ void __launch_bounds__(NT)
 __attribute__((amdgpu_waves_per_eu(HRN_WPE, HRN_WPE)))
 #endif
 hrn_mfma_kernel(const HrnKArgs a) {
-    __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE_BYTES + PF_SCRATCH];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -226,9 +252,38 @@ hrn_mfma_kernel(const HrnKArgs a) {
         }
     }
 
+    // L2 prefetch: lane -> (operand, row, line) of the tile it touches
+    uint32_t pf_off[PF_N > 0 ? PF_N : 1];
+    bool pf_isb[PF_N > 0 ? PF_N : 1];
+    if constexpr (PF > 0) {
+#pragma unroll
+        for (int i = 0; i < PF_N; ++i) {
+            const int id = i * NT + tid;                 // line id inside the tile
+            const int row = id / LPR, ln = id % LPR;
+            pf_isb[i] = (i * NT + wave * 64) / LPR >= BM;   // wave-uniform: a wave touches A or B, never both
+            const int r = pf_isb[i] ? row - BM : row;
+            const int g = (pf_isb[i] ? n0 : m0) + r;
+            const bool ok = row < BM + BN && g < (pf_isb[i] ? a.N : a.M);
+            pf_off[i] = ok ? (uint32_t)g * (uint32_t)(pf_isb[i] ? a.ldb : a.lda) * ES + ln * 128 : OOB;
+        }
+    }
+
     int issue_kt = 0;  // next k-tile to fetch
     auto issue_tile = [&](int stage) {
         char* sbase = lds + stage * STAGE_BYTES;
+        if constexpr (PF > 0) {
+            // the touched dwords are dropped into a scratch corner of LDS: no register is tied up and
+            // the loads are counted by vmcnt like the tile fetches that follow them
+            const uint32_t pk = (uint32_t)(issue_kt + PF) * BKB;
+            const bool pf_live = pk < Kb;
+            auto* scratch = (__attribute__((address_space(3))) void*)(lds + NS * STAGE_BYTES + wave * 256);
+#pragma unroll
+            for (int i = 0; i < PF_N; ++i) {
+                const uint32_t v = pf_live ? pf_off[i] + pk : OOB;
+                if (pf_isb[i]) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, scratch, 4, (int)v, 0, 0, 0);
+                else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, scratch, 4, (int)v, 0, 0, 0);
+            }
+        }
         const bool live = issue_kt < KT;
         const bool ragged = (uint32_t)(issue_kt + 1) * BKB > Kb;   // last tile not full (wave-uniform)
         const uint32_t koff = live ? (uint32_t)issue_kt * BKB : OOB;
@@ -334,13 +389,14 @@ hrn_mfma_kernel(const HrnKArgs a) {
             const int cur = kk & 1;
             if (kk == KS - 1) {
                 // every fragment of tile kt is in registers: publish tile kt+1, recycle this stage
-                wait_and_barrier<(NS - 2) * LPT, 0>();
-                issue_tile(stage);
-                read_frags(cur ^ 1, next_stage * STAGE_BYTES, 0);
+                if constexpr (ABL & 4) wait_only<(NS - 2) * LPT, 0>();
+                else wait_and_barrier<(NS - 2) * LPT, 0>();
+                if (!(ABL & 2)) issue_tile(stage);
+                if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, next_stage * STAGE_BYTES, 0);
             } else {
-                read_frags(cur ^ 1, stage_off, kk + 1);
+                if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, stage_off, kk + 1);
             }
-            mfma_step(cur);
+            if (!(ABL & 8)) mfma_step(cur);
             // pin the issue order: fragment reads (and, in the last step, the tile fetch) are
             // spread between the MFMAs of this step instead of being sunk behind them
             if (kk == KS - 1) sched_pattern<0, TM + TN, TM * TN, LPT>();

@@ -12,8 +12,8 @@ F16, U8 = B.HRN_DT_F16, B.HRN_DT_U8S8
 GEMM, CONV = B.HRN_OP_GEMM, B.HRN_OP_CONV2D
 
 
-def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0):
-    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe)
+def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, pf=0):
+    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, pf)
 
 
 # (bm, bn, bkb, wm, wn, mfma, stages, swizzle): a spread of the template space used by the parity tests
@@ -42,16 +42,19 @@ def parity_descs():
     return out
 
 
-# best known instances per benchmark workload (updated from tuning runs)
+# best known instances per benchmark workload (from CGA tuning runs on MI355X); the raster group of
+# each is in BEST_GROUP_M
 BEST = {
-    "gemm_f16": D(F16, GEMM, 256, 256, 128, 2, 2, 32, 2, 2),
-    "gemm_u8s8": D(U8, GEMM, 256, 256, 128, 2, 2, 32, 2, 2),
+    "gemm_f16": D(F16, GEMM, 256, 256, 128, 4, 2, 32, 2, 1),
+    "gemm_u8s8": D(U8, GEMM, 256, 256, 64, 2, 4, 32, 4, 3),
     "bmm_f16_qk": D(F16, GEMM, 128, 128, 128, 2, 2, 32, 2, 1),
     "bmm_f16_pv": D(F16, GEMM, 128, 64, 128, 2, 1, 32, 2, 1),
     "conv2d_f16": D(F16, CONV, 128, 64, 128, 2, 1, 32, 2, 1),
     "small": D(U8, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
     "small_f16": D(F16, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
 }
+
+BEST_GROUP_M = {"gemm_f16": 4, "gemm_u8s8": 2}
 
 
 def all_shipped():

@@ -211,7 +211,7 @@ class ldsStageOp(schedOp):
     def perform(self, s, stage_name, ctx):
         km = ctx.knob_manager
         lds_limit = ctx.getLimit('lds_bytes_per_wg')
-        stages = self.knob(ctx, stage_name, 'lds_stages', [2, 3, 4], 2)
+        stages = self.knob(ctx, stage_name, 'lds_stages', [2, 3, 4, 5], 2)
         bmn = self.var(ctx, stage_name, 'block_m_plus_n', 32, 1024, 32)
         km.addSUM(bmn, [self.V(stage_name, 'block_m'), self.V(stage_name, 'block_n')])
         sb = self.var(ctx, stage_name, 'stage_bytes', 2048, lds_limit // 2, 2048)
@@ -220,7 +220,7 @@ class ldsStageOp(schedOp):
         km.addProd([stages, sb], lds)
         if lds not in km.mems:
             km.mems.append(lds)
-        ahead = self.var(ctx, stage_name, 'stages_ahead', 1, 3, 1)
+        ahead = self.var(ctx, stage_name, 'stages_ahead', 1, 4, 1)
         km.addSUM(stages, [ahead, 1])
         inflight = self.var(ctx, stage_name, 'loads_in_flight', 1, ctx.getLimit('max_loads_in_flight'), 1)
         km.addProd([ahead, self.V(stage_name, 'loads_per_tile')], inflight)

@@ -71,11 +71,13 @@ typedef struct hrn_kernel_desc {
     int32_t bkb;        /* bytes of K per LDS stage row: 64, 128 or 256 */
     int32_t wm, wn;     /* wave grid inside the workgroup; waves = wm*wn, 64 lanes each */
     int32_t mfma;       /* 32 -> 32x32x(16 f16|32 i8), 16 -> 16x16x(32 f16|64 i8) */
-    int32_t stages;     /* LDS stages of the A/B tiles, 2..4 (2 = double buffer) */
+    int32_t stages;     /* LDS stages of the A/B tiles, 2..5 (2 = double buffer) */
     int32_t swizzle;    /* LDS 16-byte-chunk XOR swizzle: 0 none, 1 row, 2 row/2, 3 row/4 */
     int32_t epilogue;   /* 0 = store accumulators straight from registers, 1 = stage C through LDS */
     int32_t waves_per_eu; /* 0 = let the compiler pick, else occupancy hint 1..4 */
-    int32_t reserved[4];
+    int32_t l2_prefetch;  /* 0 = off, d = touch the cache lines of the k-tile d tiles past the one being fetched */
+    int32_t ablate;       /* diagnostic switches of the template; must be 0 for correct results */
+    int32_t reserved[2];
 } hrn_kernel_desc;
 
 /* Resource usage of a built instance, for cross-checks of the constraint set. */
@@ -161,6 +163,18 @@ int hrn_launch_conv2d_nhwc_f16(const hrn_module* mod, const hrn_problem* p, cons
  */
 int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C,
              int number, int repeat, double min_repeat_ms, double* costs_out, void* stream);
+
+/*
+ * Roofline probes (no counterpart in the reference, which never relates a timing to a hardware
+ * limit).  hrn_probe_mfma times a register-resident loop of independent MFMAs of the given
+ * dtype/shape on every CU and returns dense T(FL)OP/s (random_operands != 0 feeds operands with the
+ * bit statistics of real data instead of small constants: switching power lowers the sustained
+ * clock); hrn_probe_copy times a 16-byte-per-lane
+ * copy kernel over `bytes` of caller-owned device memory and returns GB/s counting read + write.
+ * The copy kernel is also the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters.
+ */
+int hrn_probe_mfma(int dtype, int mfma, int random_operands, double* tops_out, void* stream);
+int hrn_probe_copy(const void* src, void* dst, size_t bytes, int repeat, double* gbs_out, void* stream);
 
 /* Fills an hrn_problem for the plain cases (packed row-major operands). */
 void hrn_problem_gemm(hrn_problem* p, int batch, int m, int n, int k);
