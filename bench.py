@@ -56,7 +56,8 @@ def make_workloads(torch, workloads, instances):
     def build_conv():
         X, Wt = workloads.conv2d_inputs(32, 56, 56, 64, 64, 3, 3, seed=3)
         Y = torch.empty((32, 56, 56, 64), dtype=torch.float16, device="cuda")
-        return dev(X), dev(Wt), Y, B.conv2d_problem(32, 56, 56, 64, 64, 3, 3, 1, 1, 1, 8)
+        return dev(X), dev(Wt), Y, B.conv2d_problem(32, 56, 56, 64, 64, 3, 3, 1, 1, 1,
+                                                    instances.BEST_GROUP_M.get("conv2d_f16", 8))
     ops, byts = workloads.conv_work(32, 56, 56, 64, 64, 3, 3, 1, 1, 1)
     W["conv2d_f16_resnet"] = dict(desc=instances.BEST["conv2d_f16"], build=build_conv, ops=ops, bytes=byts, f16=True,
                                   desc_text="conv2d_nhwc_f16 N=32 H=W=56 C=64 K=64 3x3 s1 p1")
@@ -83,6 +84,32 @@ def measure(torch, B, w, steps, warmup):
     mod.close()
     del a, b, c
     return wall, ev, info
+
+
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
+# what the same counters read for the plain copy kernel of known size (profiles/ holds the runs these come from)
+MEASURED_TRAFFIC = {
+    "gemm_f16_4096": 244.1e6,     # profiles/hrn_mfma_kernel_gemm_f16_4096.md
+    "gemm_f16_8192": 1757e6,      # profiles/hrn_mfma_kernel_gemm_f16_8192.md
+    "gemm_u8s8_8192": 1487e6,     # profiles/hrn_mfma_kernel_gemm_u8s8_8192.md
+}
+
+
+def run_probes(torch, B):
+    """Roofline denominators measured on this GPU next to the published ones."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda")
+    dst = torch.empty(n, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    out = {
+        "mfma_f16_const_operands_TFLOPs": B.probe_mfma(B.HRN_DT_F16, 32, False, st),
+        "mfma_f16_random_operands_TFLOPs": B.probe_mfma(B.HRN_DT_F16, 32, True, st),
+        "mfma_i8_const_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 32, False, st),
+        "mfma_i8_random_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 32, True, st),
+        "hbm_copy_1GiB_read_plus_write_GBs": B.probe_copy(src.data_ptr(), dst.data_ptr(), n, 10, st),
+    }
+    del src, dst
+    return out
 
 
 def roofline(w, ev_seconds, workloads):
@@ -152,6 +179,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm_f16_4096")
     ap.add_argument("--only", action="store_true", help="skip the 'also' workloads and the CPU baseline")
+    ap.add_argument("--probe", action="store_true", help="only run the roofline probes (MFMA loop, 1 GiB copy)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the hot path is a single-GPU kernel and no multi-GPU figure is produced "
@@ -165,6 +193,9 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     B.lib()
+    if args.probe:
+        print(json.dumps({"probes": run_probes(torch, B)}))
+        return
     W = make_workloads(torch, workloads, instances)
     if args.workload not in W:
         print("unknown workload %s (have %s)" % (args.workload, sorted(W)), file=sys.stderr)
@@ -184,6 +215,10 @@ def main():
         "config": {"workload": w["desc_text"], "instance": repr(w["desc"]), "kernel_ms": ev * 1e3, "resources": info},
         "roofline": roofline(w, ev, workloads),
     }
+    line["roofline"]["traffic"] = MEASURED_TRAFFIC.get(args.workload)
+    line["peaks"] = {"published": {"mfma_f16_TFLOPs": workloads.PEAK_FP16_TFLOPS, "mfma_i8_TOPs": workloads.PEAK_INT8_TOPS,
+                                   "hbm_GBs": workloads.PEAK_HBM_GBS},
+                     "measured": run_probes(torch, B), "used": "published"}
     if not args.only:
         also = []
         for name, ww in W.items():

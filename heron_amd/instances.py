@@ -45,16 +45,16 @@ def parity_descs():
 # best known instances per benchmark workload (from CGA tuning runs on MI355X); the raster group of
 # each is in BEST_GROUP_M
 BEST = {
-    "gemm_f16": D(F16, GEMM, 256, 256, 128, 4, 2, 32, 2, 1),
+    "gemm_f16": D(F16, GEMM, 256, 256, 128, 4, 2, 32, 2, 2),
     "gemm_u8s8": D(U8, GEMM, 256, 256, 64, 2, 4, 32, 4, 3),
-    "bmm_f16_qk": D(F16, GEMM, 128, 128, 128, 2, 2, 32, 2, 1),
-    "bmm_f16_pv": D(F16, GEMM, 128, 64, 128, 2, 1, 32, 2, 1),
-    "conv2d_f16": D(F16, CONV, 128, 64, 128, 2, 1, 32, 2, 1),
+    "bmm_f16_qk": D(F16, GEMM, 128, 128, 64, 2, 4, 32, 2, 1),
+    "bmm_f16_pv": D(F16, GEMM, 64, 64, 128, 4, 2, 16, 3, 1, wpe=1),
+    "conv2d_f16": D(F16, CONV, 256, 64, 128, 2, 4, 16, 2, 1, wpe=1),
     "small": D(U8, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
     "small_f16": D(F16, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
 }
 
-BEST_GROUP_M = {"gemm_f16": 4, "gemm_u8s8": 2}
+BEST_GROUP_M = {"gemm_f16": 4, "gemm_u8s8": 2, "bmm_f16_qk": 8, "bmm_f16_pv": 2, "conv2d_f16": 2}
 
 
 def all_shipped():
