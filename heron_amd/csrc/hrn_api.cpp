@@ -36,7 +36,7 @@ struct HrnKArgs {  // must match mfma_gemm_template.hip
     int64_t sA, sB, sC;
     int32_t tiles_m, tiles_n, group_m, batch;
     int32_t H, W, CI, HO, WO, KH, KW, cstride, cpad, cdil;
-    int32_t pad0, pad1;
+    int32_t pf_sa, pf_sb;
 };
 
 struct hrn_module {
@@ -120,6 +120,8 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (d->epilogue < 0 || d->epilogue > 1) return fail(HRN_E_BADPARAM, "epilogue %d", d->epilogue);
     if (d->waves_per_eu < 0 || d->waves_per_eu > 8) return fail(HRN_E_BADPARAM, "waves_per_eu %d", d->waves_per_eu);
     if (d->l2_prefetch < 0 || d->l2_prefetch > 8) return fail(HRN_E_BADPARAM, "l2_prefetch %d not in 0..8", d->l2_prefetch);
+    if (d->load_mode < 0 || d->load_mode > 1) return fail(HRN_E_BADPARAM, "load_mode %d", d->load_mode);
+    if (d->load_mode == 1 && (d->stages != 2 || d->l2_prefetch)) return fail(HRN_E_BADPARAM, "load_mode 1 needs stages == 2 and no l2_prefetch");
     Derived r;
     r.es = d->dtype == HRN_DT_F16 ? 2 : 1;
     r.nw = d->wm * d->wn;
@@ -147,10 +149,9 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
         return fail(HRN_E_BADPARAM, "conv: swizzle period must divide rows per load round");
     {
         // every tile fetch may be preceded by the prefetch touches of a later tile
-        const int lines = (d->bm + d->bn) * ((d->bkb + 127) / 128);
         if (d->l2_prefetch && d->op != HRN_OP_GEMM) return fail(HRN_E_BADPARAM, "l2_prefetch is for GEMM only");
-        if (d->l2_prefetch && (d->bm * ((d->bkb + 127) / 128)) % 64) return fail(HRN_E_BADPARAM, "l2_prefetch needs bm*lines_per_row %% 64 == 0");
-        const int pf = d->l2_prefetch ? (lines + r.nw * 64 - 1) / (r.nw * 64) : 0;
+        if (d->l2_prefetch && r.nw < 2) return fail(HRN_E_BADPARAM, "l2_prefetch needs at least two waves");
+        const int pf = d->l2_prefetch ? 1 : 0;
         if ((d->stages - 1) * (r.lpt + pf) > 63)
             return fail(HRN_E_BADPARAM, "too many loads in flight (%d)", (d->stages - 1) * (r.lpt + pf));
     }
@@ -163,8 +164,8 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
 
 std::string desc_key(const hrn_kernel_desc* d, uint64_t srch) {
     char b[256];
-    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_a%d_f%d_%08x", d->dtype, d->op, d->bm, d->bn,
-             d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu, d->ablate, d->l2_prefetch,
+    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_a%d_f%d_l%d_%08x", d->dtype, d->op, d->bm, d->bn,
+             d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu, d->ablate, d->l2_prefetch, d->load_mode,
              (unsigned)(srch ^ (srch >> 32)));
     return b;
 }
@@ -242,6 +243,7 @@ int compile_desc(const hrn_kernel_desc* d, double timeout_s, std::string* out_pa
     def("HRN_WPE", d->waves_per_eu);
     def("HRN_ABLATE", d->ablate);   // diagnostic switches of the template, 0 in normal use
     def("HRN_PF", d->l2_prefetch);
+    def("HRN_LOAD", d->load_mode);
     args.push_back(src);
     args.push_back("-o");
     args.push_back(co_tmp);
@@ -319,6 +321,9 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
     k->tiles_m = (p->m + d.bm - 1) / d.bm;
     k->tiles_n = (p->n + d.bn - 1) / d.bn;
     k->group_m = p->group_m > 0 ? p->group_m : 8;
+    // block of tiles one XCD (32 CUs) runs at a time under the kernel's raster: pf_sb rows x pf_sa columns
+    k->pf_sb = std::max(1, std::min(k->group_m, k->tiles_m));
+    k->pf_sa = std::max(1, std::min(k->tiles_n, 32 / k->pf_sb));
     const int64_t total = (int64_t)k->tiles_m * k->tiles_n * p->batch;
     if (total <= 0 || total >= (1ll << 31)) return fail(HRN_E_BADPARAM, "grid size");
     *grid = (unsigned)total;

@@ -40,7 +40,7 @@ struct HrnKArgs {
     int32_t tiles_m, tiles_n, group_m, batch;
     // conv
     int32_t H, W, CI, HO, WO, KH, KW, cstride, cpad, cdil;
-    int32_t pad0, pad1;
+    int32_t pf_sa, pf_sb;       // L2 prefetch: column-tiles / row-tiles of the block one XCD runs concurrently
 };
 #endif
 
@@ -58,13 +58,21 @@ constexpr int EPI = HRN_EPI;
 #define HRN_ABLATE 0
 #endif
 constexpr int ABL = HRN_ABLATE;
-// L2 prefetch: with HRN_PF = d > 0 every tile fetch is preceded by one 4-byte load per 128-byte line of the
-// k-tile d tiles further on.  The data is discarded; the point is that the line is in L2 (not HBM) when the
-// real fetch arrives, because a tile is only usable when its slowest load has landed.
+// L2 prefetch: with HRN_PF = d > 0 every tile fetch is preceded by 4-byte "touch" loads of the k-tile d tiles
+// further on (this workgroup's share of the rows, see the kernel).  The data is discarded; the point is that
+// the sectors are in L2 (not HBM) when the real fetch arrives, because a tile is only usable when its slowest
+// load has landed.
 #ifndef HRN_PF
 #define HRN_PF 0
 #endif
 constexpr int PF = HRN_PF;
+// Load path: 0 = global -> LDS directly (LDS-DMA), HRN_STAGES tiles in LDS.
+//            1 = global -> registers -> LDS: two register sets hold the two tiles in flight, LDS holds the tile
+//                being multiplied and the next one (HRN_STAGES must be 2); a tile then has two tile-times to land.
+#ifndef HRN_LOAD
+#define HRN_LOAD 0
+#endif
+constexpr int LOADM = HRN_LOAD;
 constexpr int ES = (DT == 0) ? 2 : 1;       // input element bytes
 constexpr int OES = (DT == 0) ? 2 : 4;      // output element bytes
 constexpr int NW = WM * WN, NT = NW * 64;
@@ -73,7 +81,7 @@ constexpr int RPI = 64 / CPR;               // tile rows one wave load instructi
 constexpr int A_LPW = (BM / RPI) / NW;      // load instructions per wave per tile
 constexpr int B_LPW = (BN / RPI) / NW;
 constexpr int LPR = (BKB + 127) / 128;                         // 128-byte lines per tile row
-constexpr int PF_N = PF ? ((BM + BN) * LPR + NW * 64 - 1) / (NW * 64) : 0;   // prefetch touches per lane per tile
+constexpr int PF_N = PF ? 1 : 0;                                // prefetch touches per lane per tile
 constexpr int LPT = A_LPW + B_LPW + PF_N;                       // vector memory ops per lane per tile
 constexpr int KSB = (MT == 32) ? 32 : 64;   // bytes of K one MFMA consumes
 constexpr int KS = BKB / KSB;               // MFMA k-steps per tile
@@ -89,9 +97,10 @@ static_assert(MT == 32 || MT == 16, "MFMA");
 static_assert(KS >= 2 && (KS % 2) == 0, "need an even number of k-steps per tile");
 static_assert((BM / RPI) % NW == 0 && (BN / RPI) % NW == 0 && A_LPW >= 1 && B_LPW >= 1, "loads per wave");
 static_assert(OP == 0 || PF == 0, "L2 prefetch is implemented for the GEMM address pattern only");
-static_assert(PF == 0 || (BM * ((BKB + 127) / 128)) % 64 == 0, "L2 prefetch: A lines must fill whole waves");
+static_assert(PF == 0 || NW >= 2, "L2 prefetch needs one wave for each operand");
 static_assert(BM % (WM * MT) == 0 && BN % (WN * MT) == 0, "wave tile");
 static_assert(NS >= 2 && NS <= 5, "stages");
+static_assert(LOADM == 0 || (NS == 2 && PF == 0), "register-staged loads use exactly two LDS stages");
 constexpr int PF_SCRATCH = PF ? NW * 256 : 0;                   // LDS corner the prefetch touches land in
 static_assert(NS * STAGE_BYTES + PF_SCRATCH <= 163840, "LDS");
 static_assert(SWZ == 0 || (CPR << (SWZ - 1)) <= MT, "swizzle period must fit in one MFMA tile");
@@ -155,16 +164,18 @@ __device__ __forceinline__ v4i mfma(v4i x, v4i y, v4i c) {
     return __builtin_amdgcn_mfma_i32_16x16x64_i8(x, y, c, 0, 0, 0);
 }
 
-// Scheduling pattern of one k-step: NR groups of {1 LDS read, NV/NR buffer loads, NMM/NR MFMAs}.
-template <int R, int NR, int NMM, int NV>
+// Scheduling pattern of one k-step: NR groups of {1 LDS read, NV/NR buffer loads, NDW/NR LDS writes, NMM/NR MFMAs}.
+template <int R, int NR, int NMM, int NV, int NDW = 0>
 __device__ __forceinline__ void sched_pattern() {
     if constexpr (R < NR) {
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         constexpr int v = (NV * (R + 1)) / NR - (NV * R) / NR;
         if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);
+        constexpr int w = (NDW * (R + 1)) / NR - (NDW * R) / NR;
+        if constexpr (w > 0) __builtin_amdgcn_sched_group_barrier(0x200, w, 0);
         constexpr int mm = (NMM * (R + 1)) / NR - (NMM * R) / NR;
         if constexpr (mm > 0) __builtin_amdgcn_sched_group_barrier(0x008, mm, 0);
-        sched_pattern<R + 1, NR, NMM, NV>();
+        sched_pattern<R + 1, NR, NMM, NV, NDW>();
     }
 }
 
@@ -238,52 +249,46 @@ hrn_mfma_kernel(const HrnKArgs a) {
         int ke = chunk * (16 / ES);                 // element index inside K of tile 0
         cr = ke / (a.KW * a.CI); ke -= cr * (a.KW * a.CI);
         cs = ke / a.CI; cc = ke - cs * a.CI;
+        // output pixel of the lane's first row by division, of the following rows (NW*RPI further each) by carry
+        const int hw = a.HO * a.WO;
+        int m = m0 + wave * RPI + lrow;
+        int img = m / hw;
+        int rem = m - img * hw;
+        int oy = rem / a.WO, ox = rem - oy * a.WO;
 #pragma unroll
         for (int i = 0; i < A_LPW; ++i) {
-            const int row = (i * NW + wave) * RPI + lrow;
-            const int m = m0 + row;
-            const int hw = a.HO * a.WO;
-            const int img = m / hw; const int rem = m - img * hw;
-            const int oy = rem / a.WO, ox = rem - oy * a.WO;
             const bool ok = m < a.M;
             voffA[i] = (uint32_t)img * (uint32_t)(a.H * a.W * a.CI) * ES;
             iy0[i] = ok ? oy * a.cstride - a.cpad : -(1 << 28);
             ix0[i] = ox * a.cstride - a.cpad;
+            m += NW * RPI;
+            ox += NW * RPI;
+            while (ox >= a.WO) { ox -= a.WO; if (++oy == a.HO) { oy = 0; ++img; } }
         }
     }
 
-    // L2 prefetch: lane -> (operand, row, line) of the tile it touches
+    // L2 prefetch duty of this workgroup.  The tiles that run on one XCD at the same time form a block of
+    // a.pf_sb row-tiles x a.pf_sa column-tiles; the pf_sa tiles of one block row read the same rows of A and the
+    // pf_sb tiles of one block column the same rows of B, so each tile touches only its 1/pf_sa share of the A rows
+    // and 1/pf_sb share of the B rows (every 64-byte sector of them) of the k-tile PF tiles past the one being
+    // fetched.  Waves of the lower half touch A, waves of the upper half B, one touch per lane per tile.
     uint32_t pf_off[PF_N > 0 ? PF_N : 1];
-    bool pf_isb[PF_N > 0 ? PF_N : 1];
+    const bool pf_isb = wave >= (NW + 1) / 2;
     if constexpr (PF > 0) {
-#pragma unroll
-        for (int i = 0; i < PF_N; ++i) {
-            const int id = i * NT + tid;                 // line id inside the tile
-            const int row = id / LPR, ln = id % LPR;
-            pf_isb[i] = (i * NT + wave * 64) / LPR >= BM;   // wave-uniform: a wave touches A or B, never both
-            const int r = pf_isb[i] ? row - BM : row;
-            const int g = (pf_isb[i] ? n0 : m0) + r;
-            const bool ok = row < BM + BN && g < (pf_isb[i] ? a.N : a.M);
-            pf_off[i] = ok ? (uint32_t)g * (uint32_t)(pf_isb[i] ? a.ldb : a.lda) * ES + ln * 128 : OOB;
-        }
+        constexpr int SEC = BKB >= 64 ? BKB / 64 : 1;
+        const int share = pf_isb ? a.pf_sb : a.pf_sa;
+        const int duty = pf_isb ? (tin % gsz) % share : tile_n % share;
+        const int q = (pf_isb ? tid - ((NW + 1) / 2) * 64 : tid);      // touch slot inside the operand's waves
+        const int row = duty + share * (q / SEC), sec = q % SEC;
+        const int g = (pf_isb ? n0 : m0) + row;
+        const bool ok = row < (pf_isb ? BN : BM) && g < (pf_isb ? a.N : a.M);
+        pf_off[0] = ok ? (uint32_t)g * (uint32_t)(pf_isb ? a.ldb : a.lda) * ES + sec * 64 : OOB;
     }
 
     int issue_kt = 0;  // next k-tile to fetch
-    auto issue_tile = [&](int stage) {
-        char* sbase = lds + stage * STAGE_BYTES;
-        if constexpr (PF > 0) {
-            // the touched dwords are dropped into a scratch corner of LDS: no register is tied up and
-            // the loads are counted by vmcnt like the tile fetches that follow them
-            const uint32_t pk = (uint32_t)(issue_kt + PF) * BKB;
-            const bool pf_live = pk < Kb;
-            auto* scratch = (__attribute__((address_space(3))) void*)(lds + NS * STAGE_BYTES + wave * 256);
-#pragma unroll
-            for (int i = 0; i < PF_N; ++i) {
-                const uint32_t v = pf_live ? pf_off[i] + pk : OOB;
-                if (pf_isb[i]) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, scratch, 4, (int)v, 0, 0, 0);
-                else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, scratch, 4, (int)v, 0, 0, 0);
-            }
-        }
+    // Byte offsets of this lane's chunks in k-tile `issue_kt` (out-of-range offset = zeros), shared by both load paths.
+    uint32_t offA[A_LPW], offB[B_LPW];
+    auto tile_offsets = [&]() {
         const bool live = issue_kt < KT;
         const bool ragged = (uint32_t)(issue_kt + 1) * BKB > Kb;   // last tile not full (wave-uniform)
         const uint32_t koff = live ? (uint32_t)issue_kt * BKB : OOB;
@@ -296,7 +301,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
                     const uint32_t kb = koff + (uint32_t)((lpos ^ swz_of_row(row)) * 16);
                     if (kb >= Kb) v = OOB;
                 }
-                load_chunk_to_lds(rsrcA, sbase + (i * NW + wave) * 1024, v);
+                offA[i] = v;
             }
         } else {
             const int iyr = cr * a.cdil, ixs = cs * a.cdil;
@@ -305,8 +310,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
             for (int i = 0; i < A_LPW; ++i) {
                 const int iy = iy0[i] + iyr, ix = ix0[i] + ixs;
                 const bool ok = kvalid && (unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W;
-                const uint32_t v = ok ? voffA[i] + (uint32_t)((iy * a.W + ix) * a.CI + cc) * ES : OOB;
-                load_chunk_to_lds(rsrcA, sbase + (i * NW + wave) * 1024, v);
+                offA[i] = ok ? voffA[i] + (uint32_t)((iy * a.W + ix) * a.CI + cc) * ES : OOB;
             }
             // advance the lane's (kh, kw, ci) position by one k-tile
             cc += BKB / ES;
@@ -320,9 +324,49 @@ hrn_mfma_kernel(const HrnKArgs a) {
                 const uint32_t kb = koff + (uint32_t)((lpos ^ swz_of_row(row)) * 16);
                 if (kb >= Kb) v = OOB;
             }
-            load_chunk_to_lds(rsrcB, sbase + A_BYTES + (i * NW + wave) * 1024, v);
+            offB[i] = v;
         }
+    };
+
+    // path 0: fetch k-tile `issue_kt` straight into LDS stage `stage`
+    auto issue_tile = [&](int stage) {
+        char* sbase = lds + stage * STAGE_BYTES;
+        if constexpr (PF > 0) {
+            // the touched dwords are dropped into a scratch corner of LDS: no register is tied up and
+            // the loads are counted by vmcnt like the tile fetches that follow them
+            const uint32_t pk = (uint32_t)(issue_kt + PF) * BKB;
+            const bool pf_live = pk < Kb;
+            auto* scratch = (__attribute__((address_space(3))) void*)(lds + NS * STAGE_BYTES + wave * 256);
+            const uint32_t v = pf_live ? pf_off[0] + pk : OOB;
+            if (pf_isb) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, scratch, 4, (int)v, 0, 0, 0);
+            else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, scratch, 4, (int)v, 0, 0, 0);
+        }
+        tile_offsets();
+#pragma unroll
+        for (int i = 0; i < A_LPW; ++i) load_chunk_to_lds(rsrcA, sbase + (i * NW + wave) * 1024, offA[i]);
+#pragma unroll
+        for (int i = 0; i < B_LPW; ++i) load_chunk_to_lds(rsrcB, sbase + A_BYTES + (i * NW + wave) * 1024, offB[i]);
         ++issue_kt;
+    };
+
+    // path 1: fetch k-tile `issue_kt` into register set SET; later copy a set into an LDS stage
+    v4i regA[LOADM ? 2 : 1][LOADM ? A_LPW : 1], regB[LOADM ? 2 : 1][LOADM ? B_LPW : 1];
+    auto issue_regs = [&](auto setc) {
+        constexpr int SET = decltype(setc)::value;
+        tile_offsets();
+#pragma unroll
+        for (int i = 0; i < A_LPW; ++i) regA[SET][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (int)offA[i], 0, 0);
+#pragma unroll
+        for (int i = 0; i < B_LPW; ++i) regB[SET][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrcB, (int)offB[i], 0, 0);
+        ++issue_kt;
+    };
+    auto write_lds = [&](auto setc, int stage) {
+        constexpr int SET = decltype(setc)::value;
+        char* sbase = lds + stage * STAGE_BYTES + lane * 16;
+#pragma unroll
+        for (int i = 0; i < A_LPW; ++i) *(v4i*)(sbase + (i * NW + wave) * 1024) = regA[SET][i];
+#pragma unroll
+        for (int i = 0; i < B_LPW; ++i) *(v4i*)(sbase + A_BYTES + (i * NW + wave) * 1024) = regB[SET][i];
     };
 
     // ---- per-lane MFMA operand addresses ----
@@ -374,35 +418,72 @@ hrn_mfma_kernel(const HrnKArgs a) {
         }
     };
 
-    // ---- prologue: fill all stages, wait for tile 0 ----
-#pragma unroll
-    for (int s = 0; s < NS; ++s) issue_tile(s);
-    wait_and_barrier<(NS - 1) * LPT, 0>();
-    read_frags(0, 0, 0);
+    if constexpr (LOADM == 0) {
+        // ---- prologue: fill all stages, wait for tile 0 ----
+    #pragma unroll
+        for (int s = 0; s < NS; ++s) issue_tile(s);
+        wait_and_barrier<(NS - 1) * LPT, 0>();
+        read_frags(0, 0, 0);
 
-    int stage = 0;
-    for (int kt = 0; kt < KT; ++kt) {
-        const int stage_off = stage * STAGE_BYTES;
-        const int next_stage = (stage + 1 == NS) ? 0 : stage + 1;
-#pragma unroll
-        for (int kk = 0; kk < KS; ++kk) {
-            const int cur = kk & 1;
-            if (kk == KS - 1) {
-                // every fragment of tile kt is in registers: publish tile kt+1, recycle this stage
-                if constexpr (ABL & 4) wait_only<(NS - 2) * LPT, 0>();
-                else wait_and_barrier<(NS - 2) * LPT, 0>();
-                if (!(ABL & 2)) issue_tile(stage);
-                if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, next_stage * STAGE_BYTES, 0);
-            } else {
-                if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, stage_off, kk + 1);
+        int stage = 0;
+        for (int kt = 0; kt < KT; ++kt) {
+            const int stage_off = stage * STAGE_BYTES;
+            const int next_stage = (stage + 1 == NS) ? 0 : stage + 1;
+    #pragma unroll
+            for (int kk = 0; kk < KS; ++kk) {
+                const int cur = kk & 1;
+                if (kk == KS - 1) {
+                    // every fragment of tile kt is in registers: publish tile kt+1, recycle this stage
+                    if constexpr (ABL & 4) wait_only<(NS - 2) * LPT, 0>();
+                    else wait_and_barrier<(NS - 2) * LPT, 0>();
+                    if (!(ABL & 2)) issue_tile(stage);
+                    if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, next_stage * STAGE_BYTES, 0);
+                } else {
+                    if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, stage_off, kk + 1);
+                }
+                if (!(ABL & 8)) mfma_step(cur);
+                // pin the issue order: fragment reads (and, in the last step, the tile fetch) are
+                // spread between the MFMAs of this step instead of being sunk behind them
+                if (kk == KS - 1) sched_pattern<0, TM + TN, TM * TN, LPT>();
+                else sched_pattern<0, TM + TN, TM * TN, 0>();
             }
-            if (!(ABL & 8)) mfma_step(cur);
-            // pin the issue order: fragment reads (and, in the last step, the tile fetch) are
-            // spread between the MFMAs of this step instead of being sunk behind them
-            if (kk == KS - 1) sched_pattern<0, TM + TN, TM * TN, LPT>();
-            else sched_pattern<0, TM + TN, TM * TN, 0>();
+            stage = next_stage;
         }
-        stage = next_stage;
+    } else {
+        // ---- register-staged pipeline: tile t is requested during tile t-3's last k-step, copied into LDS
+        // during tile t-1 and multiplied as tile t: two tile-times for the data to arrive ----
+        using S0 = std::integral_constant<int, 0>;
+        using S1 = std::integral_constant<int, 1>;
+        issue_regs(S0{});
+        issue_regs(S1{});
+        write_lds(S0{}, 0);
+        wait_and_barrier<63, 0>();
+        issue_regs(S0{});
+        read_frags(0, 0, 0);
+        auto body = [&](auto parity) {
+            constexpr int P = decltype(parity)::value;      // LDS stage of the tile being multiplied
+            using Other = std::integral_constant<int, 1 - P>;
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) {
+                const int cur = kk & 1;
+                if (kk == KS - 2) write_lds(Other{}, 1 - P);       // next tile: registers -> the free LDS stage
+                if (kk == KS - 1) {
+                    wait_and_barrier<63, 0>();                      // LDS writes visible, old stage drained
+                    issue_regs(Other{});                            // request the tile three ahead
+                    read_frags(cur ^ 1, (1 - P) * STAGE_BYTES, 0);
+                } else {
+                    read_frags(cur ^ 1, P * STAGE_BYTES, kk + 1);
+                }
+                if (!(ABL & 8)) mfma_step(cur);
+                if (kk == KS - 1) sched_pattern<0, TM + TN, TM * TN, A_LPW + B_LPW, 0>();
+                else if (kk == KS - 2) sched_pattern<0, TM + TN, TM * TN, 0, A_LPW + B_LPW>();
+                else sched_pattern<0, TM + TN, TM * TN, 0, 0>();
+            }
+        };
+        for (int kt = 0; kt < KT; kt += 2) {
+            body(S0{});
+            if (kt + 1 < KT) body(S1{});
+        }
     }
 
     // ---- epilogue ----

@@ -12,8 +12,8 @@ F16, U8 = B.HRN_DT_F16, B.HRN_DT_U8S8
 GEMM, CONV = B.HRN_OP_GEMM, B.HRN_OP_CONV2D
 
 
-def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, pf=0):
-    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, pf)
+def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, pf=0, load=0):
+    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, pf, 0, load)
 
 
 # (bm, bn, bkb, wm, wn, mfma, stages, swizzle): a spread of the template space used by the parity tests
@@ -27,6 +27,24 @@ PARITY_SHAPES = [
     (64, 128, 256, 1, 2, 16, 2, 1),
     (32, 32, 128, 1, 2, 16, 4, 0),
 ]
+
+
+# instances that exercise the optional load paths: (tile tuple, l2_prefetch, load_mode)
+PARITY_VARIANTS = [
+    ((256, 256, 128, 4, 2, 32, 2, 2), 1, 0),
+    ((128, 128, 128, 2, 2, 32, 3, 1), 2, 0),
+    ((256, 256, 128, 4, 2, 32, 2, 2), 0, 1),
+    ((128, 64, 128, 2, 1, 16, 2, 1), 0, 1),
+]
+
+
+def variant_descs():
+    out = []
+    for t, pf, load in PARITY_VARIANTS:
+        out.append(D(F16, GEMM, *t, pf=pf, load=load))
+        out.append(D(U8, GEMM, *t, pf=pf, load=load))
+    out.append(D(F16, CONV, 128, 64, 128, 2, 1, 16, 2, 1, load=1))
+    return out
 
 
 def parity_descs():
@@ -59,7 +77,7 @@ BEST_GROUP_M = {"gemm_f16": 4, "gemm_u8s8": 2, "bmm_f16_qk": 8, "bmm_f16_pv": 2,
 
 def all_shipped():
     seen, out = set(), []
-    for d in parity_descs() + list(BEST.values()):
+    for d in parity_descs() + variant_descs() + list(BEST.values()):
         if d.as_tuple() not in seen:
             seen.add(d.as_tuple())
             out.append(d)

@@ -30,7 +30,7 @@ class TemplateSchedule:
         dtype = B.HRN_DT_F16 if self.info['kind'] == 'f16' else B.HRN_DT_U8S8
         op = B.HRN_OP_CONV2D if self.info['operator'] == 'conv2d_nhwc' else B.HRN_OP_GEMM
         return B.make_desc(dtype, op, p['bm'], p['bn'], p['bkb'], p['wm'], p['wn'], p['mfma'], p['stages'],
-                           p['swizzle'], 0, p['waves_per_eu'])
+                           p['swizzle'], 0, p['waves_per_eu'], p.get('l2_prefetch', 0))
 
     def to_problem(self):
         from ... import backend as B
@@ -222,10 +222,34 @@ class ldsStageOp(schedOp):
             km.mems.append(lds)
         ahead = self.var(ctx, stage_name, 'stages_ahead', 1, 4, 1)
         km.addSUM(stages, [ahead, 1])
+        # optional L2 prefetch: one more vector-memory op per lane and tile, at least two waves, GEMM addressing only
+        pf_cands = [0, 1, 2] if s.info['operator'] == 'gemm' else [0]
+        pf = self.knob(ctx, stage_name, 'l2_prefetch', pf_cands, 0)
+        vm_ops = self.var(ctx, stage_name, 'vmem_ops_per_tile', 2, 65, 2)
+        if len(pf_cands) > 1:
+            km.addCandidates(pf, pf_cands)
+            pf_on = self.var(ctx, stage_name, 'l2_prefetch_on', 0, 1, 0)
+            km.addSUM(1, [pf_on, pf.replace("P#", "O#") + '_cand0'])
+            km.addSUM(vm_ops, [self.V(stage_name, 'loads_per_tile'), pf_on])
+            wm1 = self.var(ctx, stage_name, 'waves_minus_1', 0, 15, 0)
+            km.addSUM(self.V(stage_name, 'waves'), [wm1, 1])
+            cap = self.var(ctx, stage_name, 'l2_prefetch_cap', 0, 30, 0)
+            km.addProd([2, wm1], cap)
+            km.addLE(pf, cap)
+            # the touched dwords land in 256 B of LDS per wave, on top of the stages
+            sw = self.var(ctx, stage_name, 'l2_prefetch_scratch_all', 256, 4096, 256)
+            km.addProd([256, self.V(stage_name, 'waves')], sw)
+            scr = self.var(ctx, stage_name, 'l2_prefetch_scratch', 0, 4096, 0)
+            km.addProd([pf_on, sw], scr)
+            total = self.var(ctx, stage_name, 'lds_bytes_total', 4096, lds_limit, 4096)
+            km.addSUM(total, [lds, scr])
+        else:
+            km.addEQ(vm_ops, self.V(stage_name, 'loads_per_tile'))
         inflight = self.var(ctx, stage_name, 'loads_in_flight', 1, ctx.getLimit('max_loads_in_flight'), 1)
-        km.addProd([ahead, self.V(stage_name, 'loads_per_tile')], inflight)
+        km.addProd([ahead, vm_ops], inflight)
         s.params['stages'] = km.get_val(stages)
-        ctx.addSchedDesc("LDS stages = %s\n" % s.params['stages'])
+        s.params['l2_prefetch'] = km.get_val(pf)
+        ctx.addSchedDesc("LDS stages = %s, L2 prefetch distance = %s\n" % (s.params['stages'], s.params['l2_prefetch']))
 
 
 class ldsSwizzleOp(schedOp):

@@ -77,7 +77,8 @@ typedef struct hrn_kernel_desc {
     int32_t waves_per_eu; /* 0 = let the compiler pick, else occupancy hint 1..4 */
     int32_t l2_prefetch;  /* 0 = off, d = touch the cache lines of the k-tile d tiles past the one being fetched */
     int32_t ablate;       /* diagnostic switches of the template; must be 0 for correct results */
-    int32_t reserved[2];
+    int32_t load_mode;    /* 0 = global -> LDS directly, 1 = global -> registers -> LDS with two tiles in flight (stages must be 2) */
+    int32_t reserved[1];
 } hrn_kernel_desc;
 
 /* Resource usage of a built instance, for cross-checks of the constraint set. */

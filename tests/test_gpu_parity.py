@@ -64,6 +64,31 @@ def test_gemm_f16_within_tolerance(tup, hrn):
         check_f16(C, oracle.gemm_f32(A, Bm))
 
 
+@pytest.mark.parametrize("desc", instances.variant_descs(), ids=lambda d: "-".join(map(str, d.as_tuple())))
+def test_optional_load_paths(desc, hrn):
+    """L2 prefetch touches and the register-staged load path must not change any result."""
+    m = mod_for(desc)
+    if desc.op == instances.CONV:
+        for i, case in enumerate(CONV_CASES[:4]):
+            N, H, W, CI, CO, KH, KW, s, p, d = case
+            X, Wt = workloads.conv2d_inputs(N, H, W, CI, CO, KH, KW, seed=40 + i)
+            print("variant conv", desc.as_tuple(), case, flush=True)
+            Y = hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, d).cpu().numpy()
+            check_f16(Y, oracle.conv2d_nhwc_f32(X, Wt, s, p, d))
+        return
+    for i, (M, K, N) in enumerate(GEMM_SHAPES + [(1024, 2048, 768)]):
+        K16 = (K + 15) // 16 * 16
+        print("variant", desc.as_tuple(), (M, K16, N), flush=True)
+        if desc.dtype == instances.U8:
+            A, Bm = workloads.gemm_u8s8_inputs(M, K16, N, seed=50 + i)
+            C = hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy()
+            assert np.array_equal(C, oracle.gemm_int64_numpy(A, Bm).astype(np.int32))
+        else:
+            A, Bm = workloads.gemm_f16_inputs(M, K16, N, seed=60 + i)
+            C = hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy()
+            check_f16(C, oracle.gemm_f32(A, Bm))
+
+
 def test_gemm_u8s8_extremes(hrn):
     """A = 255, B = -128 reaches the most negative accumulator; B = 127 the most positive."""
     m = mod_for(instances.BEST["small"])
@@ -171,6 +196,52 @@ def test_error_paths(hrn):
     mu = mod_for(instances.BEST["small"])
     with pytest.raises(ValueError):
         hostops.gemm(mu, A, A)                                           # wrong dtype for the module
+
+
+def test_hip_measurer_tunes_gemm64(hrn, tmp_path):
+    """The reference's quick-start case end to end on the GPU: 64^3 u8s8 GEMM, CGA, HIP builder + measurement
+    server, results verified against a host reference inside the measurer (Task.set_verify_func)."""
+    from heron_amd.config import Config
+    from heron_amd.environment import Env
+    from heron_amd.ops.rocm import getOpFromName
+    from heron_amd import runner as R
+    cfg = Config()
+    cfg.codegen_type, cfg.target_name, cfg.get_op = 'GPU_MFMA', 'rocm', getOpFromName
+    cfg.out_name = str(tmp_path / "OPS")
+    cfg.opt_method, cfg.max_trials, cfg.measure_time_per_round = 'CGA', 24, 8
+    cfg.pop_num, cfg.select_num, cfg.iter_walks, cfg.parallel_num = 24, 12, 2, 2
+    cfg.in_dtype, cfg.out_dtype = 'int8', 'int32'
+    runner = R.LocalRunner(number=2, repeat=3, min_repeat_ms=0, timeout=60)
+    builder = R.LocalBuilder(timeout=60, n_parallel=4)
+    try:
+        env = Env(R.measure_option(builder, runner), cfg)
+        task = env.createTask("G1", getOpFromName("gemm"), [64, 64, 64, 'int8', 'int32'], 'rocm')
+        assert env.build_kwargs['check_gpu']['lds_bytes_per_wg'] == 163840
+
+        def ref(args):
+            A, Bm = workloads.gemm_u8s8_inputs(64, 64, 64, seed=0)
+            return [A, Bm], oracle.gemm_int64_numpy(A, Bm)
+        task.set_verify_func(ref, rtol=1e-6)
+        env.tune("G1")
+        import json
+        rows = [json.loads(l) for l in open(tmp_path / "OPS" / "G1" / "records.txt")]
+        assert len(rows) >= 16 and all(r["perf"] > 0 for r in rows)         # every kernel ran and verified
+        best = max(r["perf"] for r in rows)
+        assert np.exp(-best) < 50e-6
+        s, args = task.apply_best(str(tmp_path / "OPS" / "G1" / "records.txt"))
+        assert runner.time_instance(s, args, number=2, repeat=2, min_repeat_ms=1) > 0
+        # a wrong expected output must be reported as error 100 -> perf 0
+        task.ref_output = task.ref_output + 1
+        from heron_amd.sample import Sample
+        smp = Sample(task)
+        _, point = smp.knob_manager.randSample({})
+        smp.point, smp.stmt_code = point, "wrong_" + "_".join(map(str, point))
+        env.runner.measure_batch = R.create_measure_batch(task, env.runner.measure_option)
+        env.evalSamples([smp])
+        assert smp.perf == 0.0 and not smp.valid
+    finally:
+        runner.close()
+        builder.close()
 
 
 def test_device_info_and_timing(hrn):

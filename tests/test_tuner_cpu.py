@@ -91,7 +91,7 @@ def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
     t = Task("t", getOpFromName(op), shape + [dtype, dtype], "rocm")
     t.config = cfg
     t.make_stage_schedules()
-    assert len(t.knob_manager.knob_names) == 10 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
+    assert len(t.knob_manager.knob_names) == 11 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
     seen = set()
     for _ in range(40):
         km = copy.deepcopy(t.knob_manager)
@@ -101,7 +101,10 @@ def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
         assert valid and B.check_desc(d), (d, B.lib().hrn_last_error())
         g = s.info['gemm_view']
         assert g['M'] <= math.ceil(g['M'] / d.bm) * d.bm and (16 * math.ceil(g['M'] / 16)) % d.bm == 0
-        assert B.lds_bytes(d) == km.solved_knob_vals_phenotype[[k for k in km.solver.vals if k.endswith("VA:lds_bytes")][0]]
+        vals = km.solved_knob_vals_phenotype
+        lds_key = [k for k in km.solver.vals if k.endswith("VA:lds_bytes_total")] or \
+                  [k for k in km.solver.vals if k.endswith("VA:lds_bytes")]
+        assert B.lds_bytes(d) == vals[lds_key[0]]
         assert [a.name for a in args][-1] == s.info['stage_name']
         seen.add(d.as_tuple())
     assert len(seen) > 20
