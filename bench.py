@@ -47,7 +47,7 @@ def make_workloads(torch, workloads, instances):
         W[name] = dict(desc=instances.BEST[key], build=build, ops=ops, bytes=byts, f16=f16,
                        desc_text="%s batch=%d M=%d N=%d K=%d" % ("gemm_f16" if f16 else "gemm_u8s8", batch, M, N, K))
 
-    add_gemm("gemm_f16_4096", "gemm_f16", 4096, 4096, 4096, True)
+    add_gemm("gemm_f16_4096", "gemm_f16_4096", 4096, 4096, 4096, True)
     add_gemm("gemm_f16_8192", "gemm_f16", 8192, 8192, 8192, True)
     add_gemm("gemm_u8s8_8192", "gemm_u8s8", 8192, 8192, 8192, False)
     add_gemm("bmm_f16_qk", "bmm_f16_qk", 512, 64, 512, True, 192, lambda: workloads.bmm_qk_inputs(192, 512, 64, 512))

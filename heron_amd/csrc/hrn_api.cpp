@@ -142,6 +142,14 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     r.tn = d->bn / d->wn / d->mfma;
     r.stage_bytes = (d->bm + d->bn) * d->bkb;
     r.lds = d->stages * r.stage_bytes + (d->l2_prefetch ? r.nw * 256 : 0);
+    if (d->epilogue == 1) {
+        const int oes = d->dtype == HRN_DT_F16 ? 2 : 4;
+        const int wtn = d->bn / d->wn;
+        const int base = d->dtype == HRN_DT_U8S8 ? ((d->bn * 4 + 1023) / 1024) * 1024 : 0;
+        const int epi = base + r.nw * d->mfma * (wtn * oes + 16);
+        if ((d->mfma * (wtn * oes / 16)) % 64) return fail(HRN_E_BADPARAM, "staged epilogue needs mfma*wave_tile_n*out_bytes/16 %% 64 == 0");
+        r.lds = std::max(r.lds, epi);
+    }
     if (r.lds > 163840) return fail(HRN_E_BADPARAM, "LDS %d > 163840", r.lds);
     if (d->swizzle && (r.cpr << (d->swizzle - 1)) > d->mfma)
         return fail(HRN_E_BADPARAM, "swizzle %d period %d exceeds mfma %d", d->swizzle, r.cpr << (d->swizzle - 1), d->mfma);
@@ -301,6 +309,9 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
     k->batch = p->batch;
     if ((int64_t)p->ldb * es % 16 || p->ldb < p->k) return fail(HRN_E_BADPARAM, "ldb %d", p->ldb);
     if (p->ldc % 4 || p->ldc < p->n) return fail(HRN_E_BADPARAM, "ldc %d", p->ldc);
+    if (d.epilogue == 1 && (((int64_t)p->ldc * (d.dtype == HRN_DT_F16 ? 2 : 4)) % 16 || ((uintptr_t)C % 16) ||
+                            ((int64_t)p->stride_c * (d.dtype == HRN_DT_F16 ? 2 : 4)) % 16))
+        return fail(HRN_E_BADPARAM, "the LDS-staged epilogue stores 16 bytes per lane: C, ldc and stride_c must be 16-byte aligned");
     if ((int64_t)p->n * p->ldb * es >= (1ll << 31)) return fail(HRN_E_BADPARAM, "B operand exceeds 2 GiB per batch entry");
     if (d.op == HRN_OP_GEMM) {
         if ((int64_t)p->lda * es % 16 || p->lda < p->k) return fail(HRN_E_BADPARAM, "lda %d", p->lda);

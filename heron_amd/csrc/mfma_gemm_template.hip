@@ -7,7 +7,8 @@
 //               1: conv2d NHWC x KRSC as implicit GEMM (M = n*ho*wo, N = co, K = kh*kw*ci)
 //   HRN_BM/BN   workgroup tile, HRN_BKB bytes of K per LDS row, HRN_WM x HRN_WN wave grid,
 //   HRN_MFMA    32 | 16 (MFMA tile edge), HRN_STAGES LDS stages, HRN_SWZ LDS chunk swizzle,
-//   HRN_EPI     0 register epilogue, 1 LDS-staged epilogue, HRN_WPE waves-per-SIMD hint.
+//   HRN_EPI     0 stores straight from the accumulator registers, 1 LDS-staged epilogue with 16-byte coalesced
+//               stores, HRN_WPE waves-per-SIMD hint, HRN_PF L2 prefetch distance, HRN_LOAD load path.
 //
 // Data movement: both operands are K-contiguous, so a tile is a set of rows of HRN_BKB bytes.
 // Rows are cut into 16-byte chunks; every lane moves one chunk per load straight from HBM/L2
@@ -53,7 +54,7 @@ constexpr int WM = HRN_WM, WN = HRN_WN, MT = HRN_MFMA, NS = HRN_STAGES, SWZ = HR
 constexpr int EPI = HRN_EPI;
 // Diagnostic switches for bottleneck analysis (results are WRONG when non-zero; 0 in every shipped
 // instance): 1 skip LDS fragment reads after the first tile, 2 skip global->LDS loads after the
-// prologue, 4 drop the per-tile barrier, 8 skip the MFMAs.
+// prologue, 4 drop the per-tile barrier, 8 skip the MFMAs, 16 skip the stores of C.
 #ifndef HRN_ABLATE
 #define HRN_ABLATE 0
 #endif
@@ -72,6 +73,7 @@ constexpr int PF = HRN_PF;
 #ifndef HRN_LOAD
 #define HRN_LOAD 0
 #endif
+
 constexpr int LOADM = HRN_LOAD;
 constexpr int ES = (DT == 0) ? 2 : 1;       // input element bytes
 constexpr int OES = (DT == 0) ? 2 : 4;      // output element bytes
@@ -102,7 +104,13 @@ static_assert(BM % (WM * MT) == 0 && BN % (WN * MT) == 0, "wave tile");
 static_assert(NS >= 2 && NS <= 5, "stages");
 static_assert(LOADM == 0 || (NS == 2 && PF == 0), "register-staged loads use exactly two LDS stages");
 constexpr int PF_SCRATCH = PF ? NW * 256 : 0;                   // LDS corner the prefetch touches land in
-static_assert(NS * STAGE_BYTES + PF_SCRATCH <= 163840, "LDS");
+// LDS-staged epilogue: per wave a strip of MT rows x WTN outputs, rows padded by 16 bytes; after the int8 column sums
+constexpr int EPI_PITCH = WTN * OES + 16;
+constexpr int EPI_BASE = (DT == 1) ? ((BN * 4 + 1023) / 1024) * 1024 : 0;
+constexpr int EPI_BYTES = (EPI == 1) ? EPI_BASE + NW * MT * EPI_PITCH : 0;
+constexpr int LDS_BYTES = (NS * STAGE_BYTES + PF_SCRATCH > EPI_BYTES) ? NS * STAGE_BYTES + PF_SCRATCH : EPI_BYTES;
+static_assert(LDS_BYTES <= 163840, "LDS");
+static_assert(EPI == 0 || (MT * (WTN * OES / 16)) % 64 == 0, "staged epilogue: a strip must split into whole wave stores");
 static_assert(SWZ == 0 || (CPR << (SWZ - 1)) <= MT, "swizzle period must fit in one MFMA tile");
 static_assert((NS - 1) * LPT <= 63, "vmcnt range");
 static_assert(NT <= 1024, "threads");
@@ -186,7 +194,7 @@ extern "C" __global__ void __launch_bounds__(NT)
 __attribute__((amdgpu_waves_per_eu(HRN_WPE, HRN_WPE)))
 #endif
 hrn_mfma_kernel(const HrnKArgs a) {
-    __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE_BYTES + PF_SCRATCH];
+    __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -504,6 +512,54 @@ hrn_mfma_kernel(const HrnKArgs a) {
     }
 
     char* Cb = (char*)a.C + (int64_t)bz * a.sC * OES;
+    const bool do_store = !(ABL & 16) || a.K == 0x7fffffff;   // the ablation keeps the stores reachable but never takes them
+    if constexpr (EPI == 1) {
+        // LDS-staged epilogue: a wave parks one MFMA row-tile (MT rows x WTN columns) of its result in a private,
+        // padded LDS strip, then streams it out with 16 bytes per lane, whole row segments per store instruction.
+        if constexpr (DT == 0) wait_and_barrier<0, 0>();   // (the int8 path has synchronised above) stages are dead now
+        char* strip = lds + EPI_BASE + wave * (MT * EPI_PITCH);
+        constexpr int CPRW = WTN * OES / 16;               // 16-byte chunks per strip row
+        constexpr int EPC = 16 / OES;                      // output elements per chunk
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                for (int g = 0; g < ACC_N / 4; ++g) {
+                    const int cl = j * MT + g * 8 + lq * 4;          // column inside the wave tile
+                    char* dst = strip + lr * EPI_PITCH + cl * OES;
+                    if constexpr (DT == 0) {
+                        v4h o;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[i][j][g * 4 + r];
+                        *(v4h*)dst = o;
+                    } else {
+                        const v4i bs = *(const v4i*)(bs_lds + wn_idx * WTN + cl);
+                        v4i o;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r] + 128 * bs[r];
+                        *(v4i*)dst = o;
+                    }
+                }
+            }
+            asm volatile("" ::: "memory");     // LDS serves one wave's requests in order: the reads below see the writes
+#pragma unroll
+            for (int it = 0; it < MT * CPRW / 64; ++it) {
+                const int c = it * 64 + lane;
+                const int row = c / CPRW, cc = c % CPRW;
+                const v4i val = *(const v4i*)(strip + row * EPI_PITCH + cc * 16);
+                const int m = m0 + wm_idx * WTM + i * MT + row;
+                const int n = n0 + wn_idx * WTN + cc * EPC;
+                char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
+                if (do_store && m < a.M) {
+                    if (n + EPC <= a.N) *(v4i*)dst = val;
+                    else if (DT == 0 && n + 4 <= a.N) *(long*)dst = ((long)(uint32_t)val.y << 32) | (uint32_t)val.x;
+                }
+            }
+            asm volatile("" ::: "memory");
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int m = m0 + wm_idx * WTM + i * MT + lr;
@@ -513,7 +569,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
             for (int g = 0; g < ACC_N / 4; ++g) {
                 const int nl = wn_idx * WTN + j * MT + g * 8 + lq * 4;
                 const int n = n0 + nl;
-                if (m < a.M && n < a.N) {
+                if (do_store && m < a.M && n < a.N) {
                     char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
                     if constexpr (DT == 0) {
                         v4h o;

@@ -30,6 +30,16 @@ PARITY_SHAPES = [
 
 
 # instances that exercise the optional load paths: (tile tuple, l2_prefetch, load_mode)
+# (tile tuple) instances run with the LDS-staged epilogue as well
+EPILOGUE_VARIANTS = [
+    (256, 256, 128, 4, 2, 32, 2, 2),
+    (256, 256, 64, 2, 4, 32, 4, 3),
+    (128, 128, 128, 2, 2, 32, 2, 1),
+    (64, 64, 128, 4, 2, 16, 3, 1),
+    (64, 128, 256, 1, 2, 16, 2, 1),
+    (128, 64, 128, 2, 1, 32, 2, 1),
+]
+
 PARITY_VARIANTS = [
     ((256, 256, 128, 4, 2, 32, 2, 2), 1, 0),
     ((128, 128, 128, 2, 2, 32, 3, 1), 2, 0),
@@ -44,6 +54,11 @@ def variant_descs():
         out.append(D(F16, GEMM, *t, pf=pf, load=load))
         out.append(D(U8, GEMM, *t, pf=pf, load=load))
     out.append(D(F16, CONV, 128, 64, 128, 2, 1, 16, 2, 1, load=1))
+    for t in EPILOGUE_VARIANTS:
+        out.append(D(F16, GEMM, *t, epi=1))
+        out.append(D(U8, GEMM, *t, epi=1))
+    out.append(D(F16, CONV, 256, 64, 128, 8, 1, 16, 2, 1, epi=1))
+    out.append(D(F16, CONV, 128, 64, 128, 2, 1, 32, 2, 1, epi=1))
     return out
 
 
@@ -63,16 +78,17 @@ def parity_descs():
 # best known instances per benchmark workload (from CGA tuning runs on MI355X); the raster group of
 # each is in BEST_GROUP_M
 BEST = {
-    "gemm_f16": D(F16, GEMM, 256, 256, 128, 4, 2, 32, 2, 2),
-    "gemm_u8s8": D(U8, GEMM, 256, 256, 64, 2, 4, 32, 4, 3),
-    "bmm_f16_qk": D(F16, GEMM, 128, 128, 64, 2, 4, 32, 2, 1),
-    "bmm_f16_pv": D(F16, GEMM, 64, 64, 128, 4, 2, 16, 3, 1, wpe=1),
-    "conv2d_f16": D(F16, CONV, 256, 64, 128, 2, 4, 16, 2, 1, wpe=1),
+    "gemm_f16": D(F16, GEMM, 256, 256, 128, 4, 2, 32, 2, 2, epi=1),
+    "gemm_f16_4096": D(F16, GEMM, 256, 256, 128, 2, 4, 32, 2, 2, epi=1, wpe=2),
+    "gemm_u8s8": D(U8, GEMM, 256, 256, 64, 2, 4, 32, 4, 3, epi=1),
+    "bmm_f16_qk": D(F16, GEMM, 128, 128, 64, 2, 4, 32, 2, 1, epi=1),
+    "bmm_f16_pv": D(F16, GEMM, 64, 64, 128, 4, 2, 16, 3, 1, epi=1, wpe=1),
+    "conv2d_f16": D(F16, CONV, 256, 64, 128, 8, 1, 16, 2, 1, epi=1),
     "small": D(U8, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
     "small_f16": D(F16, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
 }
 
-BEST_GROUP_M = {"gemm_f16": 4, "gemm_u8s8": 2, "bmm_f16_qk": 8, "bmm_f16_pv": 2, "conv2d_f16": 2}
+BEST_GROUP_M = {"gemm_f16": 4, "gemm_f16_4096": 4, "gemm_u8s8": 2, "bmm_f16_qk": 8, "bmm_f16_pv": 2, "conv2d_f16": 32}
 
 
 def all_shipped():

@@ -30,7 +30,7 @@ class TemplateSchedule:
         dtype = B.HRN_DT_F16 if self.info['kind'] == 'f16' else B.HRN_DT_U8S8
         op = B.HRN_OP_CONV2D if self.info['operator'] == 'conv2d_nhwc' else B.HRN_OP_GEMM
         return B.make_desc(dtype, op, p['bm'], p['bn'], p['bkb'], p['wm'], p['wn'], p['mfma'], p['stages'],
-                           p['swizzle'], 0, p['waves_per_eu'], p.get('l2_prefetch', 0))
+                           p['swizzle'], p.get('epilogue', 0), p['waves_per_eu'], p.get('l2_prefetch', 0))
 
     def to_problem(self):
         from ... import backend as B
@@ -319,6 +319,49 @@ class registerBudgetOp(schedOp):
         ctx.addSchedDesc("occupancy hint = %s\n" % s.params['waves_per_eu'])
 
 
+class epilogueOp(schedOp):
+    """Result write-back: 0 stores 8/16-byte pieces straight from the accumulator registers, 1 parks one MFMA
+    row-tile per wave in a padded LDS strip and streams it out 16 bytes per lane (whole row segments per store).
+    The strips must fit the LDS budget and split into whole wave stores.  Replaces the store stage of the reference's
+    TensorCore template (tensorcoreStoreOp through shared memory, gpu_tensorcore_operator.py), where it is not a choice."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        lds_limit = ctx.getLimit('lds_bytes_per_wg')
+        oes = 2 if s.info['kind'] == 'f16' else 4
+        epi = self.knob(ctx, stage_name, 'epilogue', [0, 1], 1)
+        wtn = self.V(stage_name, 'wave_tile_n')
+        row = self.var(ctx, stage_name, 'epi_row_bytes', 32, 1024, 64)
+        km.addProd([oes, wtn], row)
+        pitch = self.var(ctx, stage_name, 'epi_pitch', 48, 1040, 80)
+        km.addSUM(pitch, [row, 16])
+        lanes = self.var(ctx, stage_name, 'epi_rows_all', 16, 512, 32)
+        km.addProd([self.V(stage_name, 'waves'), self.P(stage_name, 'mfma')], lanes)
+        strips = self.var(ctx, stage_name, 'epi_strip_bytes', 768, lds_limit * 4, 768)
+        km.addProd([lanes, pitch], strips)
+        base = 0
+        if s.info['kind'] != 'f16':
+            base = self.var(ctx, stage_name, 'epi_base', 1024, 2048, 1024)       # column sums, rounded up to 1 KiB
+            kb = self.var(ctx, stage_name, 'epi_base_kib', 1, 2, 1)
+            km.addProd([1024, kb], base)
+            bn4 = self.var(ctx, stage_name, 'block_n_bytes4', 64, 2048, 64)
+            km.addProd([4, self.V(stage_name, 'block_n')], bn4)
+            km.addLE(bn4, base)
+        need = self.var(ctx, stage_name, 'epi_lds_needed', 768, lds_limit * 4 + 2048, 768)
+        km.addSUM(need, [strips, base])
+        used = self.var(ctx, stage_name, 'epi_lds_bytes', 0, lds_limit, 0)
+        km.addProd([epi, need], used)                       # 0 when the register epilogue is chosen
+        # a strip must split into whole 1 KiB wave stores: mfma * row_bytes = 1024 * q
+        area = self.var(ctx, stage_name, 'epi_strip_area', 512, 32768, 1024)
+        km.addProd([self.P(stage_name, 'mfma'), row], area)
+        area_e = self.var(ctx, stage_name, 'epi_strip_area_used', 0, 32768, 0)
+        km.addProd([epi, area], area_e)
+        q = self.var(ctx, stage_name, 'epi_wave_stores', 0, 32, 0)
+        km.addProd([1024, q], area_e)
+        s.params['epilogue'] = km.get_val(epi)
+        ctx.addSchedDesc("epilogue = %s\n" % s.params['epilogue'])
+
+
 class rasterOp(schedOp):
     """Launch-time tile raster: workgroups are spread over the 8 XCDs and walk the tile grid in column
     groups of ``group_m`` row-tiles so that one XCD's L2 holds a compact block of A and B."""
@@ -345,12 +388,13 @@ all_op_methods = {
     'ldsStage': ldsStageOp,
     'ldsSwizzle': ldsSwizzleOp,
     'registerBudget': registerBudgetOp,
+    'epilogue': epilogueOp,
     'raster': rasterOp,
     'finish': finishOp,
 }
 
 RULE_ORDER = ['start', 'mfmaShape', 'tileWave', 'tileBlock', 'tileK', 'loadVector', 'ldsStage', 'ldsSwizzle',
-              'registerBudget', 'raster', 'finish']
+              'registerBudget', 'epilogue', 'raster', 'finish']
 
 
 def sched_via_rule(ctx, s):
