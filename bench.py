@@ -69,12 +69,11 @@ def measure(torch, B, w, steps, warmup):
     mod = B.Module(w["desc"])
     a, b, c, prob = w["build"]()
     stream = torch.cuda.current_stream().cuda_stream
-    for _ in range(warmup):
-        mod.launch(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), stream)
+    if warmup > 0:
+        mod.launch_repeat(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), warmup, stream)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        mod.launch(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), stream)
+    mod.launch_repeat(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), steps, stream)     # exactly `steps` launches
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
     # per-launch kernel duration from HIP events recorded on the launch stream
@@ -89,9 +88,9 @@ def measure(torch, B, w, steps, warmup):
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
 # what the same counters read for the plain copy kernel of known size (profiles/ holds the runs these come from)
 MEASURED_TRAFFIC = {
-    "gemm_f16_4096": 244.1e6,     # profiles/hrn_mfma_kernel_gemm_f16_4096.md
-    "gemm_f16_8192": 1757e6,      # profiles/hrn_mfma_kernel_gemm_f16_8192.md
-    "gemm_u8s8_8192": 1487e6,     # profiles/hrn_mfma_kernel_gemm_u8s8_8192.md
+    "gemm_f16_4096": 235.0e6,     # profiles/hrn_mfma_kernel_gemm_f16_4096.md
+    "gemm_f16_8192": 1745.9e6,    # profiles/hrn_mfma_kernel_gemm_f16_8192.md
+    "gemm_u8s8_8192": 1481.9e6,   # profiles/hrn_mfma_kernel_gemm_u8s8_8192.md
 }
 
 

@@ -126,6 +126,7 @@ SYMBOLS = {
     "hrn_launch_gemm_u8s8": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
     "hrn_launch_bmm_f16": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
     "hrn_launch_conv2d_nhwc_f16": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
+    "hrn_launch_repeat": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _vp]),
     "hrn_time": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _i, _d, ctypes.POINTER(_d), _vp]),
     "hrn_problem_gemm": (None, [ctypes.POINTER(Problem), _i, _i, _i, _i]),
     "hrn_problem_conv2d": (None, [ctypes.POINTER(Problem)] + [_i] * 10),
@@ -233,6 +234,10 @@ class Module:
 
     def launch(self, problem, a_ptr, b_ptr, c_ptr, stream=0):
         _check(self._launcher(problem)(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, stream))
+
+    def launch_repeat(self, problem, a_ptr, b_ptr, c_ptr, count, stream=0):
+        """``count`` back-to-back launches issued from one host call."""
+        _check(lib().hrn_launch_repeat(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, count, stream))
 
     def time(self, problem, a_ptr, b_ptr, c_ptr, number=3, repeat=4, min_repeat_ms=0.0, stream=0):
         costs = (_d * repeat)()

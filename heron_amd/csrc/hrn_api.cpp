@@ -600,6 +600,21 @@ int hrn_launch_conv2d_nhwc_f16(const hrn_module* mod, const hrn_problem* p, cons
     return launch(mod, p, In, Filter, Out, stream);
 }
 
+int hrn_launch_repeat(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, int count,
+                      void* stream) {
+    if (count < 1) return fail(HRN_E_BADPARAM, "count %d", count);
+    HrnKArgs k;
+    unsigned grid;
+    int rc = fill_args(mod, p, A, B, C, &k, &grid);
+    if (rc) return rc;
+    size_t sz = sizeof k;
+    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &k, HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
+    for (int i = 0; i < count; ++i)
+        HIP_TRY(hipModuleLaunchKernel(mod->fn, grid, 1, 1, (unsigned)mod->info.threads, 1, 1, 0, (hipStream_t)stream,
+                                      nullptr, extra));
+    return HRN_OK;
+}
+
 int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, int number, int repeat,
              double min_repeat_ms, double* costs_out, void* stream) {
     if (!costs_out || number < 1 || repeat < 1) return fail(HRN_E_BADPARAM, "number/repeat/costs_out");

@@ -156,6 +156,11 @@ int hrn_launch_gemm_u8s8(const hrn_module* mod, const hrn_problem* p, const void
 int hrn_launch_bmm_f16(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
 int hrn_launch_conv2d_nhwc_f16(const hrn_module* mod, const hrn_problem* p, const void* In, const void* Filter, void* Out, void* stream);
 
+/* `count` back-to-back launches of the same problem from one host call (the inner loop of a time_evaluator
+ * repeat, runner/measure_methods.py:138-145, without the events). */
+int hrn_launch_repeat(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C,
+                      int count, void* stream);
+
 /*
  * Event-timed measurement with the semantics of TVM's time_evaluator as the reference uses
  * it (runner/measure_methods.py:138-145): `repeat` results, each the mean seconds of `number`
