@@ -121,16 +121,19 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (d->waves_per_eu < 0 || d->waves_per_eu > 8) return fail(HRN_E_BADPARAM, "waves_per_eu %d", d->waves_per_eu);
     if (d->l2_prefetch < 0 || d->l2_prefetch > 8) return fail(HRN_E_BADPARAM, "l2_prefetch %d not in 0..8", d->l2_prefetch);
     if (d->load_mode < 0 || d->load_mode > 1) return fail(HRN_E_BADPARAM, "load_mode %d", d->load_mode);
+    if (d->conv_window < 0 || d->conv_window > 1) return fail(HRN_E_BADPARAM, "conv_window %d", d->conv_window);
+    if (d->conv_window && (d->op != HRN_OP_CONV2D || d->load_mode || d->l2_prefetch))
+        return fail(HRN_E_BADPARAM, "conv_window is a conv2d option (load_mode 0, no l2_prefetch)");
     if (d->load_mode == 1 && (d->stages != 2 || d->l2_prefetch)) return fail(HRN_E_BADPARAM, "load_mode 1 needs stages == 2 and no l2_prefetch");
     Derived r;
     r.es = d->dtype == HRN_DT_F16 ? 2 : 1;
     r.nw = d->wm * d->wn;
     r.cpr = d->bkb / 16;
     r.rpi = 64 / r.cpr;
-    if (d->bm % r.rpi || d->bn % r.rpi || (d->bm / r.rpi) % r.nw || (d->bn / r.rpi) % r.nw)
+    if ((!d->conv_window && (d->bm % r.rpi || (d->bm / r.rpi) % r.nw)) || d->bn % r.rpi || (d->bn / r.rpi) % r.nw)
         return fail(HRN_E_BADPARAM, "tile rows must split evenly into 1 KiB wave loads (bm %d bn %d, %d rows/load, %d waves)",
                     d->bm, d->bn, r.rpi, r.nw);
-    r.a_lpw = d->bm / r.rpi / r.nw;
+    r.a_lpw = d->conv_window ? 0 : d->bm / r.rpi / r.nw;
     r.b_lpw = d->bn / r.rpi / r.nw;
     r.lpt = r.a_lpw + r.b_lpw;
     r.ksb = d->mfma == 32 ? 32 : 64;
@@ -140,7 +143,7 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
         return fail(HRN_E_BADPARAM, "tile %dx%d not divisible by wave grid %dx%d x mfma %d", d->bm, d->bn, d->wm, d->wn, d->mfma);
     r.tm = d->bm / d->wm / d->mfma;
     r.tn = d->bn / d->wn / d->mfma;
-    r.stage_bytes = (d->bm + d->bn) * d->bkb;
+    r.stage_bytes = ((d->conv_window ? 0 : d->bm) + d->bn) * d->bkb;
     r.lds = d->stages * r.stage_bytes + (d->l2_prefetch ? r.nw * 256 : 0);
     if (d->epilogue == 1) {
         const int oes = d->dtype == HRN_DT_F16 ? 2 : 4;
@@ -153,7 +156,7 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (r.lds > 163840) return fail(HRN_E_BADPARAM, "LDS %d > 163840", r.lds);
     if (d->swizzle && (r.cpr << (d->swizzle - 1)) > d->mfma)
         return fail(HRN_E_BADPARAM, "swizzle %d period %d exceeds mfma %d", d->swizzle, r.cpr << (d->swizzle - 1), d->mfma);
-    if (d->op == HRN_OP_CONV2D && d->swizzle && (r.nw * r.rpi) % (r.cpr << (d->swizzle - 1)))
+    if (d->op == HRN_OP_CONV2D && !d->conv_window && d->swizzle && (r.nw * r.rpi) % (r.cpr << (d->swizzle - 1)))
         return fail(HRN_E_BADPARAM, "conv: swizzle period must divide rows per load round");
     {
         // every tile fetch may be preceded by the prefetch touches of a later tile
@@ -172,8 +175,8 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
 
 std::string desc_key(const hrn_kernel_desc* d, uint64_t srch) {
     char b[256];
-    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_a%d_f%d_l%d_%08x", d->dtype, d->op, d->bm, d->bn,
-             d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu, d->ablate, d->l2_prefetch, d->load_mode,
+    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_a%d_f%d_l%d_c%d_%08x", d->dtype, d->op, d->bm, d->bn,
+             d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu, d->ablate, d->l2_prefetch, d->load_mode, d->conv_window,
              (unsigned)(srch ^ (srch >> 32)));
     return b;
 }
@@ -252,6 +255,7 @@ int compile_desc(const hrn_kernel_desc* d, double timeout_s, std::string* out_pa
     def("HRN_ABLATE", d->ablate);   // diagnostic switches of the template, 0 in normal use
     def("HRN_PF", d->l2_prefetch);
     def("HRN_LOAD", d->load_mode);
+    def("HRN_CONVWIN", d->conv_window);
     args.push_back(src);
     args.push_back("-o");
     args.push_back(co_tmp);
@@ -293,7 +297,8 @@ void read_info(const std::string& path, hrn_kernel_info* o) {
 }
 
 int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, HrnKArgs* k,
-              unsigned* grid) {
+              unsigned* grid, unsigned* dyn_lds) {
+    *dyn_lds = 0;
     if (!mod || !p || !A || !B || !C) return fail(HRN_E_BADPARAM, "null argument");
     const hrn_kernel_desc& d = mod->desc;
     if (p->op != d.op) return fail(HRN_E_BADPARAM, "problem op %d does not match module op %d", p->op, d.op);
@@ -328,6 +333,18 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
         if ((int64_t)p->cn * p->ch * p->cw * p->ci * es >= (1ll << 31)) return fail(HRN_E_BADPARAM, "input exceeds 2 GiB");
         k->H = p->ch; k->W = p->cw; k->CI = p->ci; k->HO = ho; k->WO = wo; k->KH = p->kh; k->KW = p->kw;
         k->cstride = p->cstride; k->cpad = p->cpad; k->cdil = p->cdil;
+        if (d.conv_window) {
+            if (p->cstride != 1 || p->cdil != 1 || ho != p->ch || wo != p->cw)
+                return fail(HRN_E_BADPARAM, "conv_window needs stride 1, dilation 1 and 'same' padding");
+            if ((p->ci * es) % d.bkb) return fail(HRN_E_BADPARAM, "conv_window needs CI*%d to be a multiple of bkb %d", es, d.bkb);
+            if (p->kh * p->kw > 32) return fail(HRN_E_BADPARAM, "conv_window supports at most 32 filter taps");
+            const int64_t rows = d.bm + 2 * (int64_t)p->cpad * (p->cw + 1);
+            const int64_t instr = (rows * (p->ci * es / 16) + 63) / 64;
+            const int64_t dyn = instr * 1024;
+            if (dyn + mod->info.lds_bytes > 163840)
+                return fail(HRN_E_BADPARAM, "conv_window: window of %lld bytes + %d static LDS exceeds 163840", (long long)dyn, mod->info.lds_bytes);
+            *dyn_lds = (unsigned)dyn;
+        }
     }
     k->tiles_m = (p->m + d.bm - 1) / d.bm;
     k->tiles_n = (p->n + d.bn - 1) / d.bn;
@@ -344,11 +361,12 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
 int launch(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream) {
     HrnKArgs k;
     unsigned grid;
-    int rc = fill_args(mod, p, A, B, C, &k, &grid);
+    unsigned dyn_lds;
+    int rc = fill_args(mod, p, A, B, C, &k, &grid, &dyn_lds);
     if (rc) return rc;
     size_t sz = sizeof k;
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &k, HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
-    HIP_TRY(hipModuleLaunchKernel(mod->fn, grid, 1, 1, (unsigned)mod->info.threads, 1, 1, 0, (hipStream_t)stream,
+    HIP_TRY(hipModuleLaunchKernel(mod->fn, grid, 1, 1, (unsigned)mod->info.threads, 1, 1, dyn_lds, (hipStream_t)stream,
                                   nullptr, extra));
     return HRN_OK;
 }
@@ -605,12 +623,13 @@ int hrn_launch_repeat(const hrn_module* mod, const hrn_problem* p, const void* A
     if (count < 1) return fail(HRN_E_BADPARAM, "count %d", count);
     HrnKArgs k;
     unsigned grid;
-    int rc = fill_args(mod, p, A, B, C, &k, &grid);
+    unsigned dyn_lds;
+    int rc = fill_args(mod, p, A, B, C, &k, &grid, &dyn_lds);
     if (rc) return rc;
     size_t sz = sizeof k;
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &k, HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
     for (int i = 0; i < count; ++i)
-        HIP_TRY(hipModuleLaunchKernel(mod->fn, grid, 1, 1, (unsigned)mod->info.threads, 1, 1, 0, (hipStream_t)stream,
+        HIP_TRY(hipModuleLaunchKernel(mod->fn, grid, 1, 1, (unsigned)mod->info.threads, 1, 1, dyn_lds, (hipStream_t)stream,
                                       nullptr, extra));
     return HRN_OK;
 }
@@ -620,7 +639,8 @@ int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const v
     if (!costs_out || number < 1 || repeat < 1) return fail(HRN_E_BADPARAM, "number/repeat/costs_out");
     HrnKArgs k;
     unsigned grid;
-    int rc = fill_args(mod, p, A, B, C, &k, &grid);
+    unsigned dyn_lds;
+    int rc = fill_args(mod, p, A, B, C, &k, &grid, &dyn_lds);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0, e1;

@@ -75,12 +75,21 @@ constexpr int PF = HRN_PF;
 #endif
 
 constexpr int LOADM = HRN_LOAD;
+// Conv window mode (HRN_OP=1, stride 1, dilation 1, 'same' padding): instead of fetching an im2col tile of A for every
+// filter tap, the workgroup loads ONCE the window of input pixels its BM output pixels can reach (a contiguous range
+// of BM + 2*pad*(W+1) pixels, all channels) and every tap reads its operand fragments from that window at a row offset
+// of r*W + s pixels; taps that fall into the padding are masked to zero in registers.  Only B (the filter) streams
+// through the LDS stages.
+#ifndef HRN_CONVWIN
+#define HRN_CONVWIN 0
+#endif
+constexpr bool CW = (HRN_CONVWIN != 0);
 constexpr int ES = (DT == 0) ? 2 : 1;       // input element bytes
 constexpr int OES = (DT == 0) ? 2 : 4;      // output element bytes
 constexpr int NW = WM * WN, NT = NW * 64;
 constexpr int CPR = BKB / 16;               // 16-byte chunks per tile row
 constexpr int RPI = 64 / CPR;               // tile rows one wave load instruction covers
-constexpr int A_LPW = (BM / RPI) / NW;      // load instructions per wave per tile
+constexpr int A_LPW = CW ? 0 : (BM / RPI) / NW;   // load instructions per wave per tile
 constexpr int B_LPW = (BN / RPI) / NW;
 constexpr int LPR = (BKB + 127) / 128;                         // 128-byte lines per tile row
 constexpr int PF_N = PF ? 1 : 0;                                // prefetch touches per lane per tile
@@ -90,14 +99,15 @@ constexpr int KS = BKB / KSB;               // MFMA k-steps per tile
 constexpr int CPS = KSB / 16;               // chunks per k-step (= 64 / MT)
 constexpr int WTM = BM / WM, WTN = BN / WN;
 constexpr int TM = WTM / MT, TN = WTN / MT;
-constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB, STAGE_BYTES = A_BYTES + B_BYTES;
+constexpr int A_BYTES = CW ? 0 : BM * BKB, B_BYTES = BN * BKB, STAGE_BYTES = A_BYTES + B_BYTES;
 constexpr int ACC_N = (MT == 32) ? 16 : 4;
 constexpr uint32_t OOB = 0x80000000u;
 
 static_assert(BKB == 64 || BKB == 128 || BKB == 256, "BKB");
 static_assert(MT == 32 || MT == 16, "MFMA");
 static_assert(KS >= 2 && (KS % 2) == 0, "need an even number of k-steps per tile");
-static_assert((BM / RPI) % NW == 0 && (BN / RPI) % NW == 0 && A_LPW >= 1 && B_LPW >= 1, "loads per wave");
+static_assert((CW || ((BM / RPI) % NW == 0 && A_LPW >= 1)) && (BN / RPI) % NW == 0 && B_LPW >= 1, "loads per wave");
+static_assert(!CW || (OP == 1 && LOADM == 0 && PF == 0), "window mode is a conv2d load path");
 static_assert(OP == 0 || PF == 0, "L2 prefetch is implemented for the GEMM address pattern only");
 static_assert(PF == 0 || NW >= 2, "L2 prefetch needs one wave for each operand");
 static_assert(BM % (WM * MT) == 0 && BN % (WN * MT) == 0, "wave tile");
@@ -239,8 +249,8 @@ hrn_mfma_kernel(const HrnKArgs a) {
         voffB[i] = (n < a.N) ? (uint32_t)n * (uint32_t)a.ldb * ES + chunk * 16 : OOB;
     }
     // GEMM: byte offset of the lane's chunk in k-tile 0.  Conv: pixel bookkeeping.
-    uint32_t voffA[A_LPW];
-    int iy0[OP == 1 ? A_LPW : 1], ix0[OP == 1 ? A_LPW : 1];
+    uint32_t voffA[(A_LPW > 0 ? A_LPW : 1)];
+    int iy0[OP == 1 ? (A_LPW > 0 ? A_LPW : 1) : 1], ix0[OP == 1 ? (A_LPW > 0 ? A_LPW : 1) : 1];
     int cc = 0, cs = 0, cr = 0;  // conv: channel / kw / kh position of the lane's chunk
     if constexpr (OP == 0) {
 #pragma unroll
@@ -250,7 +260,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
             const int m = m0 + row;
             voffA[i] = (m < a.M) ? (uint32_t)m * (uint32_t)a.lda * ES + chunk * 16 : OOB;
         }
-    } else {
+    } else if constexpr (!CW) {
         static_assert(OP == 0 || SWZ == 0 || ((NW * RPI) % (CPR << (SWZ > 0 ? SWZ - 1 : 0))) == 0,
                       "conv: the lane's chunk column must not depend on the load index");
         const int chunk = lpos ^ swz_of_row(wave * RPI + lrow);
@@ -295,7 +305,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
 
     int issue_kt = 0;  // next k-tile to fetch
     // Byte offsets of this lane's chunks in k-tile `issue_kt` (out-of-range offset = zeros), shared by both load paths.
-    uint32_t offA[A_LPW], offB[B_LPW];
+    uint32_t offA[(A_LPW > 0 ? A_LPW : 1)], offB[B_LPW];
     auto tile_offsets = [&]() {
         const bool live = issue_kt < KT;
         const bool ragged = (uint32_t)(issue_kt + 1) * BKB > Kb;   // last tile not full (wave-uniform)
@@ -311,7 +321,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
                 }
                 offA[i] = v;
             }
-        } else {
+        } else if constexpr (!CW) {
             const int iyr = cr * a.cdil, ixs = cs * a.cdil;
             const bool kvalid = live && cr < a.KH;
 #pragma unroll
@@ -358,7 +368,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
     };
 
     // path 1: fetch k-tile `issue_kt` into register set SET; later copy a set into an LDS stage
-    v4i regA[LOADM ? 2 : 1][LOADM ? A_LPW : 1], regB[LOADM ? 2 : 1][LOADM ? B_LPW : 1];
+    v4i regA[LOADM ? 2 : 1][LOADM ? (A_LPW > 0 ? A_LPW : 1) : 1], regB[LOADM ? 2 : 1][LOADM ? B_LPW : 1];
     auto issue_regs = [&](auto setc) {
         constexpr int SET = decltype(setc)::value;
         tile_offsets();
@@ -379,6 +389,50 @@ hrn_mfma_kernel(const HrnKArgs a) {
 
     // ---- per-lane MFMA operand addresses ----
     const int lr = lane % MT, lq = lane / MT;
+
+    // ---- conv window mode: the window itself (dynamic LDS) and the per-row tap masks ----
+    extern __shared__ __attribute__((aligned(1024))) char win[];
+    const int w_pitch = a.CI * ES;                       // bytes of one pixel (all channels)
+    const int w_cch = CW ? w_pitch / BKB : 1;            // k-tiles per tap
+    uint32_t tapmask[CW ? TM : 1];                       // bit t: tap t of this lane's pixel i is inside the image
+    if constexpr (CW) {
+        const int w_rows = BM + 2 * a.cpad * (a.W + 1);  // pixels the BM outputs can reach
+        const int cpp = w_pitch / 16;                    // 16-byte chunks per pixel
+        const int n_instr = (w_rows * cpp + 63) / 64;    // 1 KiB wave loads that cover the window
+        const int gp0 = m0 - a.cpad * (a.W + 1);         // input pixel index of window row 0
+        for (int q = wave; q < n_instr; q += NW) {
+            const int L = q * 64 + lane;
+            const int wrow = L / cpp, pos = L - wrow * cpp;
+            const int src = (pos & ~(CPR - 1)) | ((pos & (CPR - 1)) ^ swz_of_row(wrow));
+            const int gp = gp0 + wrow;
+            const uint32_t v = (wrow < w_rows && gp >= 0) ? (uint32_t)gp * (uint32_t)w_pitch + src * 16 : OOB;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (__attribute__((address_space(3))) void*)(win + q * 1024),
+                                                     16, (int)v, 0, 0, 0);
+        }
+        // masks: pixel of fragment row i by one division, the following rows (MT further each) by carry
+        const int hw = a.H * a.W;
+        int m = m0 + wm_idx * WTM + lr;
+        int img = m / hw;
+        int rem = m - img * hw;
+        int oy = rem / a.W, ox = rem - oy * a.W;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            uint32_t bits = 0;
+            if (m < a.M) {
+                for (int r = 0; r < a.KH; ++r)
+                    for (int s2 = 0; s2 < a.KW; ++s2) {
+                        const int iy = oy + r - a.cpad, ix = ox + s2 - a.cpad;
+                        if ((unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W) bits |= 1u << (r * a.KW + s2);
+                    }
+            }
+            tapmask[i] = bits;
+            m += MT;
+            ox += MT;
+            while (ox >= a.W) { ox -= a.W; if (++oy == a.H) { oy = 0; ++img; } }
+        }
+    }
+    const int w_lane = (wm_idx * WTM + lr);              // window mode: tile row of fragment 0
+    int rd_tap = 0, rd_cch = 0, rd_r = 0, rd_s = 0;      // window mode: tap / channel chunk of the k-tile being READ
     const int g16 = (lq ^ swz_of_row(lr)) << 4;      // swizzle period <= MT, so only lr matters
     const int a_lane = (wm_idx * WTM + lr) * BKB;
     const int b_lane = A_BYTES + (wn_idx * WTN + lr) * BKB;
@@ -398,12 +452,40 @@ hrn_mfma_kernel(const HrnKArgs a) {
     v4i fa[2][TM], fb[2][TN];
     auto read_frags = [&](int buf, int stage_off, int kk) {
         const int ko = g16 ^ (kk * KSB);
+        if constexpr (CW) {
+            const int tapoff = (rd_r < a.KH) ? rd_r * a.W + rd_s : 0;    // r*W + s pixels; 0 past the last tap
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-            fa[buf][i] = *(const v4i*)(lds + stage_off + a_lane + i * MT * BKB + ko);
+            for (int i = 0; i < TM; ++i) {
+                const int wrow = w_lane + i * MT + tapoff;
+                const int kc = (kk * CPS + lq) ^ swz_of_row(wrow);
+                fa[buf][i] = *(const v4i*)(win + wrow * w_pitch + rd_cch * BKB + kc * 16);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                fa[buf][i] = *(const v4i*)(lds + stage_off + a_lane + i * MT * BKB + ko);
+        }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
             fb[buf][j] = *(const v4i*)(lds + stage_off + b_lane + j * MT * BKB + ko);
+    };
+    // window mode: move the reader to the next k-tile (channel chunks inside a tap first, then kw, then kh)
+    auto advance_reader = [&]() {
+        if constexpr (CW) {
+            if (++rd_cch == w_cch) { rd_cch = 0; ++rd_tap; if (++rd_s == a.KW) { rd_s = 0; ++rd_r; } }
+        }
+    };
+    int mm_tap = 0, mm_cch = 0;                           // window mode: tap of the k-tile being MULTIPLIED
+    v4i amask[CW ? TM : 1];
+    auto set_masks = [&]() {
+        if constexpr (CW) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int on = -(int)((tapmask[i] >> mm_tap) & 1u);
+                amask[i] = (v4i){on, on, on, on};
+            }
+            if (++mm_cch == w_cch) { mm_cch = 0; ++mm_tap; }
+        }
     };
     auto mfma_step = [&](int buf) {
         if constexpr (DT == 1) {
@@ -420,6 +502,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             v4i av = fa[buf][i];
+            if constexpr (CW) av = av & amask[i];               // taps in the padding contribute zero
             if constexpr (DT == 1) av = av ^ (int)0x80808080;   // u8 -> s8 by subtracting 128
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j] = mfma(fb[buf][j], av, acc[i][j]);
@@ -437,6 +520,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
         for (int kt = 0; kt < KT; ++kt) {
             const int stage_off = stage * STAGE_BYTES;
             const int next_stage = (stage + 1 == NS) ? 0 : stage + 1;
+            set_masks();
     #pragma unroll
             for (int kk = 0; kk < KS; ++kk) {
                 const int cur = kk & 1;
@@ -445,6 +529,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
                     if constexpr (ABL & 4) wait_only<(NS - 2) * LPT, 0>();
                     else wait_and_barrier<(NS - 2) * LPT, 0>();
                     if (!(ABL & 2)) issue_tile(stage);
+                    advance_reader();
                     if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, next_stage * STAGE_BYTES, 0);
                 } else {
                     if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, stage_off, kk + 1);

@@ -12,8 +12,8 @@ F16, U8 = B.HRN_DT_F16, B.HRN_DT_U8S8
 GEMM, CONV = B.HRN_OP_GEMM, B.HRN_OP_CONV2D
 
 
-def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, pf=0, load=0):
-    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, pf, 0, load)
+def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, pf=0, load=0, win=0):
+    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, pf, 0, load, win)
 
 
 # (bm, bn, bkb, wm, wn, mfma, stages, swizzle): a spread of the template space used by the parity tests
@@ -58,6 +58,9 @@ def variant_descs():
         out.append(D(F16, GEMM, *t, epi=1))
         out.append(D(U8, GEMM, *t, epi=1))
     out.append(D(F16, CONV, 256, 64, 128, 8, 1, 16, 2, 1, epi=1))
+    out.append(D(F16, CONV, 256, 64, 128, 8, 1, 16, 2, 1, epi=1, win=1))
+    out.append(D(F16, CONV, 128, 64, 128, 2, 2, 32, 3, 1, win=1))
+    out.append(D(F16, CONV, 64, 64, 64, 2, 2, 32, 2, 2, epi=1, win=1))
     out.append(D(F16, CONV, 128, 64, 128, 2, 1, 32, 2, 1, epi=1))
     return out
 
@@ -83,7 +86,7 @@ BEST = {
     "gemm_u8s8": D(U8, GEMM, 256, 256, 64, 2, 4, 32, 4, 3, epi=1),
     "bmm_f16_qk": D(F16, GEMM, 128, 128, 64, 2, 4, 32, 2, 1, epi=1),
     "bmm_f16_pv": D(F16, GEMM, 64, 64, 128, 4, 2, 16, 3, 1, epi=1, wpe=1),
-    "conv2d_f16": D(F16, CONV, 256, 64, 128, 8, 1, 16, 2, 1, epi=1),
+    "conv2d_f16": D(F16, CONV, 256, 64, 128, 8, 1, 16, 2, 1, epi=1, win=1),
     "small": D(U8, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
     "small_f16": D(F16, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
 }

@@ -30,7 +30,8 @@ class TemplateSchedule:
         dtype = B.HRN_DT_F16 if self.info['kind'] == 'f16' else B.HRN_DT_U8S8
         op = B.HRN_OP_CONV2D if self.info['operator'] == 'conv2d_nhwc' else B.HRN_OP_GEMM
         return B.make_desc(dtype, op, p['bm'], p['bn'], p['bkb'], p['wm'], p['wn'], p['mfma'], p['stages'],
-                           p['swizzle'], p.get('epilogue', 0), p['waves_per_eu'], p.get('l2_prefetch', 0))
+                           p['swizzle'], p.get('epilogue', 0), p['waves_per_eu'], p.get('l2_prefetch', 0), 0, 0,
+                           p.get('conv_window', 0))
 
     def to_problem(self):
         from ... import backend as B
@@ -179,6 +180,43 @@ class tileKOp(schedOp):
         ctx.addSchedDesc("k tile = %s bytes\n" % s.params['bkb'])
 
 
+class convWindowOp(schedOp):
+    """conv2d only: 1 keeps the window of input pixels the tile's outputs can reach (bm + 2*pad*(W+1) pixels, all
+    channels) in LDS and reads every filter tap from it; 0 fetches an im2col tile of A per tap.  Window mode needs
+    stride 1, dilation 1, 'same' padding, at most 32 taps and whole k-tiles per pixel (CI*2 = q * bkb).  It plays the
+    role of the reference's compute_at choice for the padded-input stage (GPUfinishOp position knobs,
+    gpu_common.py:154-223): where the shared copy of the input lives relative to the reduction loops."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        ok = False
+        pitch = 16
+        halo = 0
+        if s.info['operator'] == 'conv2d_nhwc':
+            c = s.info['conv']
+            ok = (c['stride'] == 1 and c['dil'] == 1 and c['HO'] == c['H'] and c['WO'] == c['W'] and c['KH'] * c['KW'] <= 32)
+            pitch = c['CI'] * 2
+            halo = 2 * c['pad'] * (c['W'] + 1)
+        win = self.knob(ctx, stage_name, 'conv_window', [0, 1] if ok else [0], 1 if ok else 0)
+        staged = self.var(ctx, stage_name, 'a_rows_staged', 0, 512, 16)       # rows of A that go through the stages
+        off = self.var(ctx, stage_name, 'conv_window_off', 0, 1, 1)
+        km.addSUM(1, [win, off])
+        km.addProd([off, self.V(stage_name, 'block_m')], staged)
+        # window bytes (0 when off) and whole k-tiles per pixel
+        rows = self.var(ctx, stage_name, 'window_rows', 16, 512 + halo, 16 + halo)
+        km.addSUM(rows, [self.V(stage_name, 'block_m'), halo])
+        wb = self.var(ctx, stage_name, 'window_bytes_full', 256, (512 + halo) * pitch, 256)
+        km.addProd([pitch, rows], wb)
+        used = self.var(ctx, stage_name, 'window_bytes', 0, ctx.getLimit('lds_bytes_per_wg'), 0)
+        km.addProd([win, wb], used)
+        pw = self.var(ctx, stage_name, 'window_pitch_used', 0, pitch, 0)
+        km.addProd([win, pitch], pw)
+        q = self.var(ctx, stage_name, 'window_k_tiles_per_pixel', 0, max(1, pitch // 64), 0)
+        km.addProd([q, self.P(stage_name, 'block_k_bytes')], pw)
+        s.params['conv_window'] = km.get_val(win)
+        ctx.addSchedDesc("conv window mode = %s\n" % s.params['conv_window'])
+
+
 class loadVectorOp(schedOp):
     """Global->LDS transfer: every lane moves one 128-bit chunk per load and one wave instruction fills
     1 KiB of LDS, so a tile must split into whole wave loads: bm = loads_a * (64/chunks_per_row) * waves.
@@ -212,12 +250,15 @@ class ldsStageOp(schedOp):
         km = ctx.knob_manager
         lds_limit = ctx.getLimit('lds_bytes_per_wg')
         stages = self.knob(ctx, stage_name, 'lds_stages', [2, 3, 4, 5], 2)
-        bmn = self.var(ctx, stage_name, 'block_m_plus_n', 32, 1024, 32)
-        km.addSUM(bmn, [self.V(stage_name, 'block_m'), self.V(stage_name, 'block_n')])
-        sb = self.var(ctx, stage_name, 'stage_bytes', 2048, lds_limit // 2, 2048)
+        bmn = self.var(ctx, stage_name, 'block_m_plus_n', 16, 1024, 32)
+        km.addSUM(bmn, [self.V(stage_name, 'a_rows_staged'), self.V(stage_name, 'block_n')])
+        sb = self.var(ctx, stage_name, 'stage_bytes', 1024, lds_limit // 2, 2048)
         km.addProd([bmn, self.P(stage_name, 'block_k_bytes')], sb)
-        lds = self.var(ctx, stage_name, 'lds_bytes', 4096, lds_limit, 4096)
+        lds = self.var(ctx, stage_name, 'lds_bytes', 2048, lds_limit, 4096)
         km.addProd([stages, sb], lds)
+        # the conv window (dynamic LDS, rounded up to whole 1 KiB wave loads) shares the budget
+        with_win = self.var(ctx, stage_name, 'lds_bytes_with_window', 2048, lds_limit - 1024, 4096)
+        km.addSUM(with_win, [lds, self.V(stage_name, 'window_bytes')])
         if lds not in km.mems:
             km.mems.append(lds)
         ahead = self.var(ctx, stage_name, 'stages_ahead', 1, 4, 1)
@@ -384,6 +425,7 @@ all_op_methods = {
     'tileWave': tileWaveOp,
     'tileBlock': tileBlockOp,
     'tileK': tileKOp,
+    'convWindow': convWindowOp,
     'loadVector': loadVectorOp,
     'ldsStage': ldsStageOp,
     'ldsSwizzle': ldsSwizzleOp,
@@ -393,7 +435,7 @@ all_op_methods = {
     'finish': finishOp,
 }
 
-RULE_ORDER = ['start', 'mfmaShape', 'tileWave', 'tileBlock', 'tileK', 'loadVector', 'ldsStage', 'ldsSwizzle',
+RULE_ORDER = ['start', 'mfmaShape', 'tileWave', 'tileBlock', 'tileK', 'convWindow', 'loadVector', 'ldsStage', 'ldsSwizzle',
               'registerBudget', 'epilogue', 'raster', 'finish']
 
 

@@ -78,7 +78,8 @@ typedef struct hrn_kernel_desc {
     int32_t l2_prefetch;  /* 0 = off, d = touch the cache lines of the k-tile d tiles past the one being fetched */
     int32_t ablate;       /* diagnostic switches of the template; must be 0 for correct results */
     int32_t load_mode;    /* 0 = global -> LDS directly, 1 = global -> registers -> LDS with two tiles in flight (stages must be 2) */
-    int32_t reserved[1];
+    int32_t conv_window;  /* conv2d only: 1 = keep the reachable input window in LDS and read every filter tap from it
+                             (needs stride 1, dilation 1, 'same' padding, CI*2 a multiple of bkb) instead of im2col tiles */
 } hrn_kernel_desc;
 
 /* Resource usage of a built instance, for cross-checks of the constraint set. */

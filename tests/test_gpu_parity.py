@@ -68,6 +68,23 @@ def test_gemm_f16_within_tolerance(tup, hrn):
 def test_optional_load_paths(desc, hrn):
     """L2 prefetch touches and the register-staged load path must not change any result."""
     m = mod_for(desc)
+    if desc.op == instances.CONV and desc.conv_window:
+        same = [(2, 14, 14, 64, 64, 3, 3, 1, 1, 1), (1, 9, 11, 64, 32, 3, 3, 1, 1, 1), (2, 8, 8, 64, 48, 1, 1, 1, 0, 1),
+                (3, 7, 7, 128, 64, 5, 5, 1, 2, 1), (2, 56, 56, 64, 64, 3, 3, 1, 1, 1)]
+        for i, case in enumerate(same):
+            N, H, W, CI, CO, KH, KW, s, p, d = case
+            X, Wt = workloads.conv2d_inputs(N, H, W, CI, CO, KH, KW, seed=70 + i)
+            print("window conv", desc.as_tuple(), case, flush=True)
+            Y = hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, d).cpu().numpy()
+            check_f16(Y, oracle.conv2d_nhwc_f32(X, Wt, s, p, d))
+        # shapes the window path cannot serve are refused, not mis-computed
+        for case in [(1, 15, 15, 64, 16, 3, 3, 2, 1, 1), (1, 12, 12, 64, 8, 3, 3, 1, 2, 2), (1, 9, 9, 64, 8, 3, 3, 1, 0, 1),
+                     (1, 5, 600, 128, 16, 3, 3, 1, 1, 1)]:
+            N, H, W, CI, CO, KH, KW, s, p, d = case
+            X, Wt = workloads.conv2d_inputs(N, H, W, CI, CO, KH, KW, seed=1)
+            with pytest.raises(B.HeronRocmError):
+                hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, d)
+        return
     if desc.op == instances.CONV:
         for i, case in enumerate(CONV_CASES[:4]):
             N, H, W, CI, CO, KH, KW, s, p, d = case

@@ -91,7 +91,7 @@ def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
     t = Task("t", getOpFromName(op), shape + [dtype, dtype], "rocm")
     t.config = cfg
     t.make_stage_schedules()
-    assert len(t.knob_manager.knob_names) == 12 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
+    assert len(t.knob_manager.knob_names) == 13 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
     seen = set()
     for _ in range(40):
         km = copy.deepcopy(t.knob_manager)
@@ -105,7 +105,10 @@ def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
         lds_key = [k for k in km.solver.vals if k.endswith("VA:lds_bytes_total")] or \
                   [k for k in km.solver.vals if k.endswith("VA:lds_bytes")]
         epi_key = [k for k in km.solver.vals if k.endswith("VA:epi_lds_bytes")][0]
-        assert B.lds_bytes(d) == max(vals[lds_key[0]], vals[epi_key])
+        assert B.lds_bytes(d) == max(vals[lds_key[0]], vals[epi_key])         # static LDS; the conv window is dynamic
+        if op == "c2d" and d.conv_window:
+            win_key = [k for k in km.solver.vals if k.endswith("VA:window_bytes")][0]
+            assert vals[win_key] == (d.bm + 2 * (56 + 1)) * 128 and B.lds_bytes(d) + vals[win_key] <= 163840 - 1024
         assert [a.name for a in args][-1] == s.info['stage_name']
         seen.add(d.as_tuple())
     assert len(seen) > 20
