@@ -126,6 +126,8 @@ SYMBOLS = {
     "hrn_launch_gemm_u8s8": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
     "hrn_launch_bmm_f16": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
     "hrn_launch_conv2d_nhwc_f16": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
+    "hrn_launch_bmm_u8s8": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
+    "hrn_launch_conv2d_nhwc_u8s8": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
     "hrn_launch_repeat": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _vp]),
     "hrn_time": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _i, _d, ctypes.POINTER(_d), _vp]),
     "hrn_problem_gemm": (None, [ctypes.POINTER(Problem), _i, _i, _i, _i]),
@@ -227,9 +229,9 @@ class Module:
     def _launcher(self, problem):
         L = lib()
         if self.desc.op == HRN_OP_CONV2D:
-            return L.hrn_launch_conv2d_nhwc_f16
+            return L.hrn_launch_conv2d_nhwc_u8s8 if self.desc.dtype == HRN_DT_U8S8 else L.hrn_launch_conv2d_nhwc_f16
         if self.desc.dtype == HRN_DT_U8S8:
-            return L.hrn_launch_gemm_u8s8
+            return L.hrn_launch_bmm_u8s8 if problem.batch > 1 else L.hrn_launch_gemm_u8s8
         return L.hrn_launch_bmm_f16 if problem.batch > 1 else L.hrn_launch_gemm_f16
 
     def launch(self, problem, a_ptr, b_ptr, c_ptr, stream=0):

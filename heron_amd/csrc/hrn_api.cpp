@@ -110,7 +110,6 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (!d) return fail(HRN_E_BADPARAM, "null descriptor");
     if (d->dtype != HRN_DT_F16 && d->dtype != HRN_DT_U8S8) return fail(HRN_E_BADPARAM, "dtype %d", d->dtype);
     if (d->op != HRN_OP_GEMM && d->op != HRN_OP_CONV2D) return fail(HRN_E_BADPARAM, "op %d", d->op);
-    if (d->op == HRN_OP_CONV2D && d->dtype != HRN_DT_F16) return fail(HRN_E_BADPARAM, "conv2d is fp16 only");
     if (d->bkb != 64 && d->bkb != 128 && d->bkb != 256) return fail(HRN_E_BADPARAM, "bkb %d not in {64,128,256}", d->bkb);
     if (d->mfma != 32 && d->mfma != 16) return fail(HRN_E_BADPARAM, "mfma %d not in {16,32}", d->mfma);
     if (d->wm < 1 || d->wn < 1 || d->wm * d->wn > 16) return fail(HRN_E_BADPARAM, "wave grid %dx%d", d->wm, d->wn);
@@ -605,6 +604,7 @@ int hrn_launch_gemm_f16(const hrn_module* mod, const hrn_problem* p, const void*
 
 int hrn_launch_gemm_u8s8(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream) {
     if (mod && (mod->desc.dtype != HRN_DT_U8S8 || mod->desc.op != HRN_OP_GEMM)) return fail(HRN_E_BADPARAM, "module is not a u8s8 GEMM");
+    if (p && p->batch != 1) return fail(HRN_E_BADPARAM, "gemm takes batch 1 (use hrn_launch_bmm_u8s8)");
     return launch(mod, p, A, B, C, stream);
 }
 
@@ -615,6 +615,16 @@ int hrn_launch_bmm_f16(const hrn_module* mod, const hrn_problem* p, const void* 
 
 int hrn_launch_conv2d_nhwc_f16(const hrn_module* mod, const hrn_problem* p, const void* In, const void* Filter, void* Out, void* stream) {
     if (mod && (mod->desc.dtype != HRN_DT_F16 || mod->desc.op != HRN_OP_CONV2D)) return fail(HRN_E_BADPARAM, "module is not an fp16 conv2d");
+    return launch(mod, p, In, Filter, Out, stream);
+}
+
+int hrn_launch_bmm_u8s8(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream) {
+    if (mod && (mod->desc.dtype != HRN_DT_U8S8 || mod->desc.op != HRN_OP_GEMM)) return fail(HRN_E_BADPARAM, "module is not a u8s8 GEMM");
+    return launch(mod, p, A, B, C, stream);
+}
+
+int hrn_launch_conv2d_nhwc_u8s8(const hrn_module* mod, const hrn_problem* p, const void* In, const void* Filter, void* Out, void* stream) {
+    if (mod && (mod->desc.dtype != HRN_DT_U8S8 || mod->desc.op != HRN_OP_CONV2D)) return fail(HRN_E_BADPARAM, "module is not a u8s8 conv2d");
     return launch(mod, p, In, Filter, Out, stream);
 }
 

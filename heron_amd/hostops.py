@@ -34,10 +34,20 @@ def gemm(mod, A, Bm, out=None, group_m=8):
     return out
 
 
+def unpack_filter_blocked(Wb):
+    """Blocked int8 filter (CO/b,KH,KW,CI/4,b,4) of ops/x86/conv2d_int8.py:50 -> KRSC (CO,KH,KW,CI); a one-off
+    reorder of the weights on the device."""
+    OC, KH, KW, ICC, cb, four = Wb.shape
+    if four != 4:
+        raise ValueError("expected (CO/b,KH,KW,CI/4,b,4), got %s" % (tuple(Wb.shape),))
+    return Wb.permute(0, 4, 1, 2, 3, 5).reshape(OC * cb, KH, KW, ICC * 4).contiguous()
+
+
 def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8):
-    """X (N,H,W,CI) fp16, Wt KRSC (CO,KH,KW,CI) fp16 -> (N,HO,WO,CO) fp16."""
-    _chk(X, torch.float16)
-    _chk(Wt, torch.float16)
+    """X (N,H,W,CI), Wt KRSC (CO,KH,KW,CI) -> (N,HO,WO,CO): fp16 -> fp16, or uint8 x int8 -> int32."""
+    f16 = mod.desc.dtype == B.HRN_DT_F16
+    _chk(X, torch.float16 if f16 else torch.uint8)
+    _chk(Wt, torch.float16 if f16 else torch.int8)
     N, H, W, CI = X.shape
     CO, KH, KW, CI2 = Wt.shape
     if CI != CI2:
@@ -46,6 +56,6 @@ def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8):
     ho = (H - ((KH - 1) * dil + 1) + 2 * pad) // stride + 1
     wo = (W - ((KW - 1) * dil + 1) + 2 * pad) // stride + 1
     if out is None:
-        out = torch.empty((N, ho, wo, CO), dtype=torch.float16, device=X.device)
+        out = torch.empty((N, ho, wo, CO), dtype=torch.float16 if f16 else torch.int32, device=X.device)
     mod.launch(p, X.data_ptr(), Wt.data_ptr(), out.data_ptr(), _stream())
     return out

@@ -78,6 +78,18 @@ def parity_descs():
     return out
 
 
+def int8_conv_descs():
+    """uint8 x int8 -> int32 conv2d instances of the parity suite (im2col and window load paths)."""
+    return [
+        D(U8, CONV, 64, 64, 64, 2, 2, 32, 2, 1),
+        D(U8, CONV, 128, 64, 128, 2, 2, 16, 3, 1, epi=1),
+        D(U8, CONV, 128, 128, 128, 2, 2, 32, 2, 1, epi=1),
+        D(U8, CONV, 64, 32, 128, 2, 1, 16, 4, 0),
+        D(U8, CONV, 128, 64, 64, 4, 1, 32, 2, 1, epi=1, win=1),
+        D(U8, CONV, 256, 64, 128, 8, 1, 16, 2, 1, win=1),
+    ]
+
+
 # best known instances per benchmark workload (from CGA tuning runs on MI355X); the raster group of
 # each is in BEST_GROUP_M
 BEST = {
@@ -96,7 +108,7 @@ BEST_GROUP_M = {"gemm_f16": 4, "gemm_f16_4096": 4, "gemm_u8s8": 2, "bmm_f16_qk":
 
 def all_shipped():
     seen, out = set(), []
-    for d in parity_descs() + variant_descs() + list(BEST.values()):
+    for d in parity_descs() + variant_descs() + int8_conv_descs() + list(BEST.values()):
         if d.as_tuple() not in seen:
             seen.add(d.as_tuple())
             out.append(d)

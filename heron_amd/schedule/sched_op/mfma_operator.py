@@ -183,7 +183,7 @@ class tileKOp(schedOp):
 class convWindowOp(schedOp):
     """conv2d only: 1 keeps the window of input pixels the tile's outputs can reach (bm + 2*pad*(W+1) pixels, all
     channels) in LDS and reads every filter tap from it; 0 fetches an im2col tile of A per tap.  Window mode needs
-    stride 1, dilation 1, 'same' padding, at most 32 taps and whole k-tiles per pixel (CI*2 = q * bkb).  It plays the
+    stride 1, dilation 1, 'same' padding, at most 32 taps and whole k-tiles per pixel (CI*elem_bytes = q * bkb).  It plays the
     role of the reference's compute_at choice for the padded-input stage (GPUfinishOp position knobs,
     gpu_common.py:154-223): where the shared copy of the input lives relative to the reduction loops."""
 
@@ -195,7 +195,7 @@ class convWindowOp(schedOp):
         if s.info['operator'] == 'conv2d_nhwc':
             c = s.info['conv']
             ok = (c['stride'] == 1 and c['dil'] == 1 and c['HO'] == c['H'] and c['WO'] == c['W'] and c['KH'] * c['KW'] <= 32)
-            pitch = c['CI'] * 2
+            pitch = c['CI'] * (2 if s.info['kind'] == 'f16' else 1)
             halo = 2 * c['pad'] * (c['W'] + 1)
         win = self.knob(ctx, stage_name, 'conv_window', [0, 1] if ok else [0], 1 if ok else 0)
         staged = self.var(ctx, stage_name, 'a_rows_staged', 0, 512, 16)       # rows of A that go through the stages
@@ -388,6 +388,9 @@ class epilogueOp(schedOp):
             bn4 = self.var(ctx, stage_name, 'block_n_bytes4', 64, 2048, 64)
             km.addProd([4, self.V(stage_name, 'block_n')], bn4)
             km.addLE(bn4, base)
+            slack = self.var(ctx, stage_name, 'block_n_bytes4_plus_1023', 1087, 3071, 1087)
+            km.addSUM(slack, [bn4, 1023])
+            km.addLE(base, slack)                               # base is the smallest whole KiB that holds the sums
         need = self.var(ctx, stage_name, 'epi_lds_needed', 768, lds_limit * 4 + 2048, 768)
         km.addSUM(need, [strips, base])
         used = self.var(ctx, stage_name, 'epi_lds_bytes', 0, lds_limit, 0)

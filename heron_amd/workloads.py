@@ -49,6 +49,14 @@ def conv2d_inputs(N, H, W, CI, CO, KH, KW, seed=3):
     return X, Wt
 
 
+def conv2d_u8s8_inputs(N, H, W, CI, CO, KH, KW, seed=6):
+    """uint8 NHWC activations and int8 KRSC weights over their full ranges (ops/x86/conv2d_int8.py:51-52)."""
+    rng = np.random.default_rng(seed)
+    X = rng.integers(0, 256, (N, H, W, CI), dtype=np.uint8)
+    Wt = rng.integers(-128, 128, (CO, KH, KW, CI), dtype=np.int8)
+    return X, Wt
+
+
 def conv_out_hw(H, W, KH, KW, stride, pad, dil):
     """Output size formula of ops/cuda/conv2d.py:168-175."""
     ho = (H - ((KH - 1) * dil + 1) + 2 * pad) // stride + 1

@@ -151,11 +151,17 @@ int hrn_lds_bytes(const hrn_kernel_desc* desc);
  *   hrn_launch_gemm_u8s8       ops/x86/dense.py:6-32           (uint8 x int8 -> int32)
  *   hrn_launch_bmm_f16         ops/cuda/batch_matmul.py:5-56
  *   hrn_launch_conv2d_nhwc_f16 ops/cuda/conv2d.py:137-232      (filter KRSC)
+ *   hrn_launch_bmm_u8s8        ops/x86/batch_matmul.py:6-34    (uint8 x int8 -> int32 per batch entry)
+ *   hrn_launch_conv2d_nhwc_u8s8 ops/x86/conv2d_int8.py:31-109  (uint8 NHWC input, int8 filter -> int32; the filter is
+ *                              taken KRSC (co,kh,kw,ci), not in the reference's blocked (co/b,kh,kw,ci/4,b,4) order;
+ *                              the output (n,ho,wo,co) is the reference's (n,ho,wo,co/b,b) seen flat)
  */
 int hrn_launch_gemm_f16(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
 int hrn_launch_gemm_u8s8(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
 int hrn_launch_bmm_f16(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
 int hrn_launch_conv2d_nhwc_f16(const hrn_module* mod, const hrn_problem* p, const void* In, const void* Filter, void* Out, void* stream);
+int hrn_launch_bmm_u8s8(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
+int hrn_launch_conv2d_nhwc_u8s8(const hrn_module* mod, const hrn_problem* p, const void* In, const void* Filter, void* Out, void* stream);
 
 /* `count` back-to-back launches of the same problem from one host call (the inner loop of a time_evaluator
  * repeat, runner/measure_methods.py:138-145, without the events). */

@@ -15,6 +15,9 @@
  *   orc_bmm_u8s8s32_scalar    ops/x86/batch_matmul.py:6-34
  *   orc_gemm_f32              ops/cuda/dense.py:4-54       C[i,j] = sum_k A[i,k] * B[j,k]   (B stored (N,K))
  *   orc_bmm_f32               ops/cuda/batch_matmul.py:5-56
+ *   orc_conv2d_nhwc_u8s8s32   ops/x86/conv2d_int8.py:31-109  (filter KRSC, output (N,HO,WO,CO))
+ *   orc_conv2d_nhwc_u8s8s32_blocked  the same operator with the reference's own operand shapes: filter
+ *                             (CO/b, KH, KW, CI/4, b, 4), output (N,HO,WO,CO/b,b)   (conv2d_int8.py:50-93)
  *   orc_conv2d_nhwc_f32       ops/cuda/conv2d.py:137-232   (filter taken as KRSC = (CO,KH,KW,CI); the
  *                             reference stores HWIO (KH,KW,CI,CO) - same sum, different weight order)
  *
@@ -246,4 +249,73 @@ ORC_API void orc_conv2d_nhwc_f32(const float* In, const float* Wt, float* Out,
                     }
                     Out[((n * HO + y) * WO + x) * CO + f] = (float)acc;
                 }
+}
+
+/*
+ * ops/x86/conv2d_int8.py:74-93 with the filter in KRSC order.  uint8 input, int8 filter, int32 sum;
+ * the padding value is 0 (conv2d_int8.py:68-72 pads with the dtype's zero).
+ */
+ORC_API void orc_conv2d_nhwc_u8s8s32(const uint8_t* In, const int8_t* Wt, int32_t* Out,
+                                     int64_t N, int64_t H, int64_t W, int64_t CI, int64_t CO,
+                                     int64_t KH, int64_t KW, int64_t stride, int64_t pad, int64_t dil) {
+    const int64_t HO = (H - ((KH - 1) * dil + 1) + 2 * pad) / stride + 1;
+    const int64_t WO = (W - ((KW - 1) * dil + 1) + 2 * pad) / stride + 1;
+#pragma omp parallel for collapse(3) schedule(static)
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t y = 0; y < HO; ++y)
+            for (int64_t x = 0; x < WO; ++x)
+                for (int64_t f = 0; f < CO; ++f) {
+                    int32_t acc = 0;
+                    for (int64_t ry = 0; ry < KH; ++ry) {
+                        const int64_t iy = y * stride + ry * dil - pad;
+                        if (iy < 0 || iy >= H) continue;
+                        for (int64_t rx = 0; rx < KW; ++rx) {
+                            const int64_t ix = x * stride + rx * dil - pad;
+                            if (ix < 0 || ix >= W) continue;
+                            const uint8_t* a = In + ((n * H + iy) * W + ix) * CI;
+                            const int8_t* w = Wt + ((f * KH + ry) * KW + rx) * CI;
+                            for (int64_t c = 0; c < CI; ++c) acc += (int32_t)a[c] * (int32_t)w[c];
+                        }
+                    }
+                    Out[((n * HO + y) * WO + x) * CO + f] = acc;
+                }
+}
+
+/*
+ * The operator with the reference's operand shapes (conv2d_int8.py:50-52,74-93): filter
+ * (CO/cb, KH, KW, CI/4, cb, 4) for w_format "OhwI<cb>o4i", output (N, HO, WO, CO/cb, cb); the loop
+ * nest and index expressions are those of the te.compute, with the padded input formed explicitly.
+ */
+ORC_API int orc_conv2d_nhwc_u8s8s32_blocked(const uint8_t* In, const int8_t* Wb, int32_t* Out,
+                                            int64_t N, int64_t H, int64_t W, int64_t CI, int64_t CO,
+                                            int64_t KH, int64_t KW, int64_t stride, int64_t pad, int64_t dil,
+                                            int64_t cb) {
+    if (cb <= 0 || CO % cb || CI % 4) return -1;
+    const int64_t HO = (H - ((KH - 1) * dil + 1) + 2 * pad) / stride + 1;
+    const int64_t WO = (W - ((KW - 1) * dil + 1) + 2 * pad) / stride + 1;
+    const int64_t HP = H + 2 * pad, WP = W + 2 * pad;
+    uint8_t* P = (uint8_t*)calloc((size_t)(N * HP * WP * CI), 1);
+    if (!P) return -2;
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t y = 0; y < H; ++y)
+            memcpy(P + ((n * HP + y + pad) * WP + pad) * CI, In + (n * H + y) * W * CI, (size_t)(W * CI));
+    const int64_t ICC = CI / 4;
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t yy = 0; yy < HO; ++yy)
+            for (int64_t xx = 0; xx < WO; ++xx)
+                for (int64_t occ = 0; occ < CO / cb; ++occ)
+                    for (int64_t ocb = 0; ocb < cb; ++ocb) {
+                        int32_t acc = 0;
+                        for (int64_t ry = 0; ry < KH; ++ry)
+                            for (int64_t rx = 0; rx < KW; ++rx)
+                                for (int64_t icc = 0; icc < ICC; ++icc)
+                                    for (int64_t icb = 0; icb < 4; ++icb) {
+                                        const int32_t a = P[((n * HP + yy * stride + ry * dil) * WP + xx * stride + rx * dil) * CI + icc * 4 + icb];
+                                        const int32_t w = Wb[((((occ * KH + ry) * KW + rx) * ICC + icc) * cb + ocb) * 4 + icb];
+                                        acc += a * w;
+                                    }
+                        Out[(((n * HO + yy) * WO + xx) * (CO / cb) + occ) * cb + ocb] = acc;
+                    }
+    free(P);
+    return 0;
 }

@@ -52,6 +52,9 @@ def lib():
         L.orc_gemm_f32.argtypes = [_p, _p, _p, _i64, _i64, _i64]
         L.orc_bmm_f32.argtypes = [_p, _p, _p, _i64, _i64, _i64, _i64]
         L.orc_conv2d_nhwc_f32.argtypes = [_p, _p, _p] + [_i64] * 10
+        L.orc_conv2d_nhwc_u8s8s32.argtypes = [_p, _p, _p] + [_i64] * 10
+        L.orc_conv2d_nhwc_u8s8s32_blocked.argtypes = [_p, _p, _p] + [_i64] * 11
+        L.orc_conv2d_nhwc_u8s8s32_blocked.restype = ctypes.c_int
         _lib = L
     return _lib
 
@@ -164,6 +167,56 @@ def conv2d_nhwc_f32(In, Wt, stride=1, pad=0, dil=1):
     Out = np.empty((N, HO, WO, CO), np.float32)
     lib().orc_conv2d_nhwc_f32(_ptr(In), _ptr(Wt), _ptr(Out), N, H, W, CI, CO, KH, KW, stride, pad, dil)
     return Out
+
+
+def conv2d_nhwc_u8s8s32(In, Wt, stride=1, pad=0, dil=1):
+    """In (N,H,W,CI) uint8, Wt KRSC (CO,KH,KW,CI) int8 -> (N,HO,WO,CO) int32."""
+    In = _c(In, np.uint8); Wt = _c(Wt, np.int8)
+    N, H, W, CI = In.shape; CO, KH, KW, CI2 = Wt.shape
+    assert CI == CI2
+    HO = conv_out_size(H, KH, stride, pad, dil); WO = conv_out_size(W, KW, stride, pad, dil)
+    Out = np.empty((N, HO, WO, CO), np.int32)
+    lib().orc_conv2d_nhwc_u8s8s32(_ptr(In), _ptr(Wt), _ptr(Out), N, H, W, CI, CO, KH, KW, stride, pad, dil)
+    return Out
+
+
+def conv2d_nhwc_u8s8s32_blocked(In, Wb, stride=1, pad=0, dil=1):
+    """The reference's operand shapes: Wb (CO/cb,KH,KW,CI/4,cb,4) int8 -> (N,HO,WO,CO/cb,cb) int32."""
+    In = _c(In, np.uint8); Wb = _c(Wb, np.int8)
+    N, H, W, CI = In.shape; OC, KH, KW, ICC, cb, four = Wb.shape
+    assert four == 4 and ICC * 4 == CI
+    CO = OC * cb
+    HO = conv_out_size(H, KH, stride, pad, dil); WO = conv_out_size(W, KW, stride, pad, dil)
+    Out = np.empty((N, HO, WO, OC, cb), np.int32)
+    rc = lib().orc_conv2d_nhwc_u8s8s32_blocked(_ptr(In), _ptr(Wb), _ptr(Out), N, H, W, CI, CO, KH, KW, stride, pad, dil, cb)
+    assert rc == 0
+    return Out
+
+
+def pack_filter_blocked(Wt, cb):
+    """KRSC (CO,KH,KW,CI) -> the reference's "OhwI<cb>o4i" order (CO/cb,KH,KW,CI/4,cb,4) (conv2d_int8.py:36-50)."""
+    CO, KH, KW, CI = Wt.shape
+    assert CO % cb == 0 and CI % 4 == 0
+    return np.ascontiguousarray(Wt.reshape(CO // cb, cb, KH, KW, CI // 4, 4).transpose(0, 2, 3, 4, 1, 5))
+
+
+def unpack_filter_blocked(Wb):
+    OC, KH, KW, ICC, cb, four = Wb.shape
+    return np.ascontiguousarray(Wb.transpose(0, 4, 1, 2, 3, 5).reshape(OC * cb, KH, KW, ICC * 4))
+
+
+def conv2d_im2col_int64_numpy(In, Wt, stride=1, pad=0, dil=1):
+    """Closed form: explicit im2col matrix (numpy indexing) times the flattened filter, in int64."""
+    N, H, W, CI = In.shape; CO, KH, KW, _ = Wt.shape
+    HO = conv_out_size(H, KH, stride, pad, dil); WO = conv_out_size(W, KW, stride, pad, dil)
+    P = np.zeros((N, H + 2 * pad, W + 2 * pad, CI), np.int64)
+    P[:, pad:pad + H, pad:pad + W, :] = In
+    cols = np.empty((N, HO, WO, KH, KW, CI), np.int64)
+    for ry in range(KH):
+        for rx in range(KW):
+            cols[:, :, :, ry, rx, :] = P[:, ry * dil:ry * dil + (HO - 1) * stride + 1:stride,
+                                         rx * dil:rx * dil + (WO - 1) * stride + 1:stride, :]
+    return (cols.reshape(N * HO * WO, KH * KW * CI) @ Wt.astype(np.int64).reshape(CO, -1).T).reshape(N, HO, WO, CO)
 
 
 def gemm_f64_numpy(A, B):

@@ -32,21 +32,42 @@ def makeConfig(args):
     return config
 
 
+def _im2col(X, KH, KW, stride, pad, dil):
+    N, H, W, CI = X.shape
+    HO = (H - ((KH - 1) * dil + 1) + 2 * pad) // stride + 1
+    WO = (W - ((KW - 1) * dil + 1) + 2 * pad) // stride + 1
+    P = np.zeros((N, H + 2 * pad, W + 2 * pad, CI), X.dtype)
+    P[:, pad:pad + H, pad:pad + W, :] = X
+    cols = np.empty((N, HO, WO, KH, KW, CI), X.dtype)
+    for ry in range(KH):
+        for rx in range(KW):
+            cols[:, :, :, ry, rx, :] = P[:, ry * dil:ry * dil + (HO - 1) * stride + 1:stride,
+                                         rx * dil:rx * dil + (WO - 1) * stride + 1:stride, :]
+    return cols.reshape(N * HO * WO, KH * KW * CI), (N, HO, WO)
+
+
 def host_reference(op_name):
-    """numpy reference for --check: returns func(args) -> ([inputs], expected_output)."""
-    def gemm(params):
-        *shape, in_dtype, _ = params
+    """numpy reference for --check: returns func(params) -> ([inputs], expected_output)."""
+    def ref(params):
+        shape = [x for x in params[:-2] if not isinstance(x, str)]     # drop a w_format entry
+        f16 = params[-2] == "float16"
+        wide = np.float32 if f16 else np.int64
         if op_name == "gemm":
             M, K, N = shape
-            if in_dtype == "float16":
-                A, B = workloads.gemm_f16_inputs(M, K, N)
-                return [A, B], (A.astype(np.float32) @ B.astype(np.float32).T)
-            A, B = workloads.gemm_u8s8_inputs(M, K, N)
-            return [A, B], (A.astype(np.int64) @ B.astype(np.int64).T)
-        b, M, K, N = shape
-        A, B = workloads.bmm_qk_inputs(b, M, K, N)
-        return [A, B], np.einsum("bik,bjk->bij", A.astype(np.float32), B.astype(np.float32))
-    return gemm
+            A, B = workloads.gemm_f16_inputs(M, K, N) if f16 else workloads.gemm_u8s8_inputs(M, K, N)
+            return [A, B], A.astype(wide) @ B.astype(wide).T
+        if op_name == "bmm":
+            b, M, K, N = shape
+            if f16:
+                A, B = workloads.bmm_qk_inputs(b, M, K, N)
+            else:
+                A, B = (np.stack(t) for t in zip(*[workloads.gemm_u8s8_inputs(M, K, N, seed=i) for i in range(b)]))
+            return [A, B], np.einsum("bik,bjk->bij", A.astype(wide), B.astype(wide))
+        N, H, W, CI, CO, KH, KW, stride, pad, dil = shape
+        X, Wt = (workloads.conv2d_inputs if f16 else workloads.conv2d_u8s8_inputs)(N, H, W, CI, CO, KH, KW)
+        cols, oshape = _im2col(X.astype(wide), KH, KW, stride, pad, dil)
+        return [X, Wt], (cols @ Wt.astype(wide).reshape(CO, -1).T).reshape(*oshape, CO)
+    return ref
 
 
 def run(op_name, task_name, params, env, runner, check=False):
@@ -54,7 +75,7 @@ def run(op_name, task_name, params, env, runner, check=False):
     op = config.get_op(op_name)
     task = env.createTask(task_name, op, params, config.target_name)
     task.device_id = config.device_id
-    if check and op_name in ("gemm", "bmm"):
+    if check and op_name in ("gemm", "bmm", "c2d", "c2d_nhwc"):
         task.set_verify_func(host_reference(op_name), rtol=1e-2)
     if config.tuned == "":
         env.tune(task_name)

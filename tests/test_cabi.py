@@ -40,7 +40,7 @@ def test_check_desc_mirrors_template_constraints():
         instances.D(instances.F16, instances.GEMM, 256, 256, 64, 2, 2, 16, 2, 0),     # one k-step per tile
         instances.D(instances.F16, instances.GEMM, 96, 128, 128, 2, 2, 32, 2, 0),     # 96 rows / (2 waves x 32)
         instances.D(instances.F16, instances.GEMM, 128, 128, 256, 2, 2, 16, 2, 2),    # swizzle period 32 > mfma 16
-        instances.D(instances.U8, instances.CONV, 128, 128, 128, 2, 2, 32, 2, 1),     # conv is fp16 only
+        instances.D(instances.F16, instances.GEMM, 128, 128, 128, 2, 2, 32, 2, 1, win=1),   # window mode is a conv load path
         instances.D(instances.F16, instances.GEMM, 512, 512, 64, 2, 2, 32, 2, 0),     # 1024 accumulators
         instances.D(instances.F16, instances.GEMM, 128, 128, 128, 8, 4, 32, 2, 0),    # 32 waves
     ]

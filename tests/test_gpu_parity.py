@@ -189,6 +189,54 @@ def test_conv2d_nhwc_f16(tup, hrn):
         check_f16(Y, oracle.conv2d_nhwc_f32(X, Wt, s, p, d))
 
 
+INT8_CONV_CASES = [
+    # N, H, W, CI, CO, KH, KW, stride, pad, dil      (CI a multiple of 16: whole 16-byte channel chunks)
+    (2, 14, 14, 64, 64, 3, 3, 1, 1, 1),
+    (1, 9, 11, 16, 32, 3, 3, 1, 1, 1),
+    (2, 8, 8, 32, 48, 1, 1, 1, 0, 1),
+    (1, 15, 15, 16, 16, 3, 3, 2, 1, 1),
+    (1, 12, 12, 48, 8, 3, 3, 1, 2, 2),
+    (3, 7, 7, 128, 64, 5, 5, 1, 2, 1),
+]
+
+
+@pytest.mark.parametrize("desc", instances.int8_conv_descs(), ids=lambda d: "-".join(map(str, d.as_tuple())))
+def test_conv2d_nhwc_u8s8_bit_exact(desc, hrn):
+    m = mod_for(desc)
+    ran = 0
+    for i, case in enumerate(INT8_CONV_CASES):
+        N, H, W, CI, CO, KH, KW, s, p, d = case
+        X, Wt = workloads.conv2d_u8s8_inputs(N, H, W, CI, CO, KH, KW, seed=90 + i)
+        print("int8 conv", desc.as_tuple(), case, flush=True)
+        if desc.conv_window and (s != 1 or d != 1 or 2 * p != (KH - 1) or CI % desc.bkb):
+            with pytest.raises(B.HeronRocmError):
+                hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, d)
+            continue
+        Y = hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, d).cpu().numpy()
+        assert Y.dtype == np.int32 and np.array_equal(Y, oracle.conv2d_nhwc_u8s8s32(X, Wt, s, p, d))
+        ran += 1
+    assert ran >= 1
+
+
+def test_conv2d_u8s8_extremes_and_blocked_filter(hrn):
+    """255 x -128 on every tap (largest magnitude the int32 sum sees) and weights handed over in the
+    blocked (CO/b,KH,KW,CI/4,b,4) order of the x86 operator, reordered once on the device."""
+    m = mod_for(instances.int8_conv_descs()[1])
+    X = np.full((1, 6, 6, 64), 255, np.uint8)
+    Wt = np.full((64, 3, 3, 64), -128, np.int8)
+    Y = hostops.conv2d_nhwc(m, dev(X), dev(Wt), 1, 1, 1).cpu().numpy()
+    assert Y[0, 2, 2, 0] == 9 * 64 * 255 * -128 and Y[0, 0, 0, 63] == 4 * 64 * 255 * -128
+    assert np.array_equal(Y, oracle.conv2d_nhwc_u8s8s32(X, Wt, 1, 1, 1))
+    X, Wt = workloads.conv2d_u8s8_inputs(2, 9, 9, 32, 96, 3, 3, seed=8)
+    for cb in (32, 48):
+        Wb = oracle.pack_filter_blocked(Wt, cb)
+        Wk = hostops.unpack_filter_blocked(dev(Wb))
+        assert np.array_equal(Wk.cpu().numpy(), Wt)
+        Y = hostops.conv2d_nhwc(m, dev(X), Wk, 2, 1, 1).cpu().numpy()
+        ref = oracle.conv2d_nhwc_u8s8s32_blocked(X, Wb, 2, 1, 1)              # (N,HO,WO,CO/cb,cb)
+        assert np.array_equal(Y.reshape(ref.shape), ref)
+
+
 def test_conv_1x1_is_gemm(hrn):
     """A 1x1 convolution is the GEMM of the flattened pixels: both templates must agree bit for bit."""
     tup = instances.PARITY_SHAPES[2]

@@ -117,6 +117,74 @@ def test_conv_1x1_reduces_to_gemm():
     assert np.array_equal(got, ref)
 
 
+def brute_conv(X, Wt, s, p, d):
+    N, H, W, CI = X.shape
+    CO, KH, KW, _ = Wt.shape
+    HO, WO = workloads.conv_out_hw(H, W, KH, KW, s, p, d)
+    out = np.zeros((N, HO, WO, CO), np.int64)
+    for n in range(N):
+        for y in range(HO):
+            for x in range(WO):
+                for f in range(CO):
+                    acc = 0
+                    for ry in range(KH):
+                        for rx in range(KW):
+                            iy, ix = y * s + ry * d - p, x * s + rx * d - p
+                            if 0 <= iy < H and 0 <= ix < W:
+                                for c in range(CI):
+                                    acc += int(X[n, iy, ix, c]) * int(Wt[f, ry, rx, c])
+                    out[n, y, x, f] = acc
+    return out
+
+
+INT_CONV = [(1, 5, 6, 4, 3, 3, 3, 1, 1, 1), (2, 6, 5, 8, 4, 3, 2, 2, 1, 1), (1, 7, 7, 4, 2, 3, 3, 1, 2, 2),
+            (1, 4, 4, 16, 5, 1, 1, 1, 0, 1)]
+
+
+@pytest.mark.parametrize("case", INT_CONV)
+def test_int_conv_against_brute_force_im2col_and_torch(case):
+    N, H, W, CI, CO, KH, KW, s, p, d = case
+    X, Wt = workloads.conv2d_u8s8_inputs(N, H, W, CI, CO, KH, KW, seed=sum(case))
+    got = oracle.conv2d_nhwc_u8s8s32(X, Wt, s, p, d)
+    assert got.dtype == np.int32
+    assert np.array_equal(got, brute_conv(X, Wt, s, p, d))                    # python loops
+    assert np.array_equal(got, oracle.conv2d_im2col_int64_numpy(X, Wt, s, p, d))   # explicit im2col matrix, int64
+    x = torch.from_numpy(X.astype(np.float64)).permute(0, 3, 1, 2)
+    w = torch.from_numpy(Wt.astype(np.float64)).permute(0, 3, 1, 2)
+    ref = torch.nn.functional.conv2d(x, w, stride=s, padding=p, dilation=d).permute(0, 2, 3, 1).numpy()
+    assert np.array_equal(got, ref.astype(np.int64))                           # library routine, exact in float64
+
+
+def test_int_conv_unsigned_input_signed_filter_and_extremes():
+    # 255 * -128 over every tap: interior pixels reach KH*KW*CI*255*-128, corners see only 4 of the 9 taps
+    X = np.full((1, 5, 5, 16), 255, np.uint8)
+    Wt = np.full((2, 3, 3, 16), -128, np.int8)
+    got = oracle.conv2d_nhwc_u8s8s32(X, Wt, 1, 1, 1)
+    assert got[0, 2, 2, 0] == 9 * 16 * 255 * -128 and got[0, 0, 0, 1] == 4 * 16 * 255 * -128
+    # the input is unsigned: 200 must not be read as -56
+    X = np.full((1, 1, 1, 4), 200, np.uint8)
+    Wt = np.ones((1, 1, 1, 4), np.int8)
+    assert oracle.conv2d_nhwc_u8s8s32(X, Wt)[0, 0, 0, 0] == 800
+
+
+@pytest.mark.parametrize("cb", [32, 48, 64])
+def test_int_conv_blocked_operands_equal_krsc(cb):
+    """The reference's blocked filter (CO/cb,KH,KW,CI/4,cb,4) and 5-d output against the KRSC/NHWC form."""
+    CO, CI = 2 * cb, 8
+    X, Wt = workloads.conv2d_u8s8_inputs(1, 6, 7, CI, CO, 3, 3, seed=cb)
+    Wb = oracle.pack_filter_blocked(Wt, cb)
+    assert Wb.shape == (2, 3, 3, 2, cb, 4)
+    # the packing itself, element by element: Wb[oc, r, s, ic, ob, ib] = Wt[oc*cb+ob, r, s, ic*4+ib]
+    rng = np.random.default_rng(1)
+    for _ in range(50):
+        oc, r, s_, ic, ob, ib = (int(rng.integers(0, n)) for n in Wb.shape)
+        assert Wb[oc, r, s_, ic, ob, ib] == Wt[oc * cb + ob, r, s_, ic * 4 + ib]
+    assert np.array_equal(oracle.unpack_filter_blocked(Wb), Wt)
+    got = oracle.conv2d_nhwc_u8s8s32_blocked(X, Wb, 2, 1, 1)
+    assert got.shape == (1, 3, 4, 2, cb)
+    assert np.array_equal(got.reshape(1, 3, 4, CO), oracle.conv2d_nhwc_u8s8s32(X, Wt, 2, 1, 1))
+
+
 def test_workload_generators_are_seeded_and_shaped():
     A1, B1 = workloads.gemm_u8s8_inputs(64, 64, 64, seed=0)
     A2, B2 = workloads.gemm_u8s8_inputs(64, 64, 64, seed=0)

@@ -83,7 +83,9 @@ def make_env(tmp_path, method="CGA", trials=48, case=("gemm", [1024, 1024, 1024]
 
 @pytest.mark.parametrize("op,shape,dtype", [("gemm", [8192, 8192, 8192], "float16"), ("gemm", [64, 64, 64], "int8"),
                                             ("bmm", [192, 512, 64, 512], "float16"),
-                                            ("c2d", [32, 56, 56, 64, 64, 3, 3, 1, 1, 1], "float16")])
+                                            ("c2d", [32, 56, 56, 64, 64, 3, 3, 1, 1, 1], "float16"),
+                                            ("c2d", [32, 56, 56, 64, 64, 3, 3, 1, 1, 1, "OhwI64o4i"], "int8"),
+                                            ("bmm", [12, 512, 64, 512], "int8")])
 def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
     """The Python constraint set and hrn_check_desc describe the same template space."""
     cfg = Config()
@@ -108,7 +110,7 @@ def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
         assert B.lds_bytes(d) == max(vals[lds_key[0]], vals[epi_key])         # static LDS; the conv window is dynamic
         if op == "c2d" and d.conv_window:
             win_key = [k for k in km.solver.vals if k.endswith("VA:window_bytes")][0]
-            assert vals[win_key] == (d.bm + 2 * (56 + 1)) * 128 and B.lds_bytes(d) + vals[win_key] <= 163840 - 1024
+            assert vals[win_key] == (d.bm + 2 * (56 + 1)) * (128 if dtype == "float16" else 64) and B.lds_bytes(d) + vals[win_key] <= 163840 - 1024
         assert [a.name for a in args][-1] == s.info['stage_name']
         seen.add(d.as_tuple())
     assert len(seen) > 20
