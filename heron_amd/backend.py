@@ -79,7 +79,8 @@ class Problem(ctypes.Structure):
                 ("cn", ctypes.c_int32), ("ch", ctypes.c_int32), ("cw", ctypes.c_int32), ("ci", ctypes.c_int32),
                 ("co", ctypes.c_int32), ("kh", ctypes.c_int32), ("kw", ctypes.c_int32),
                 ("cstride", ctypes.c_int32), ("cpad", ctypes.c_int32), ("cdil", ctypes.c_int32),
-                ("group_m", ctypes.c_int32), ("reserved", ctypes.c_int32 * 3)]
+                ("group_m", ctypes.c_int32),
+                ("cstride_w", ctypes.c_int32), ("cpad_w", ctypes.c_int32), ("cdil_w", ctypes.c_int32)]
 
 
 def make_desc(dtype, op=HRN_OP_GEMM, bm=128, bn=128, bkb=128, wm=2, wn=2, mfma=32, stages=2, swizzle=1,
@@ -132,6 +133,7 @@ SYMBOLS = {
     "hrn_time": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _i, _d, ctypes.POINTER(_d), _vp]),
     "hrn_problem_gemm": (None, [ctypes.POINTER(Problem), _i, _i, _i, _i]),
     "hrn_problem_conv2d": (None, [ctypes.POINTER(Problem)] + [_i] * 10),
+    "hrn_problem_conv2d_hw": (None, [ctypes.POINTER(Problem)] + [_i] * 13),
     "hrn_probe_mfma": (_i, [_i, _i, _i, ctypes.POINTER(_d), _vp]),
     "hrn_probe_copy": (_i, [_vp, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_last_error": (ctypes.c_char_p, []),
@@ -193,9 +195,15 @@ def gemm_problem(batch, m, n, k, group_m=8):
     return p
 
 
+def _pair(v):
+    return (int(v), int(v)) if isinstance(v, int) else (int(v[0]), int(v[1]))
+
+
 def conv2d_problem(n, h, w, ci, co, kh, kw, stride, pad, dil, group_m=8):
+    """``stride``, ``pad`` and ``dil`` are ints or (height, width) pairs."""
     p = Problem()
-    lib().hrn_problem_conv2d(ctypes.byref(p), n, h, w, ci, co, kh, kw, stride, pad, dil)
+    (sh, sw), (ph, pw), (dh, dw) = _pair(stride), _pair(pad), _pair(dil)
+    lib().hrn_problem_conv2d_hw(ctypes.byref(p), n, h, w, ci, co, kh, kw, sh, sw, ph, pw, dh, dw)
     p.group_m = group_m
     return p
 

@@ -37,6 +37,7 @@ struct HrnKArgs {  // must match mfma_gemm_template.hip
     int32_t tiles_m, tiles_n, group_m, batch;
     int32_t H, W, CI, HO, WO, KH, KW, cstride, cpad, cdil;
     int32_t pf_sa, pf_sb;
+    int32_t cstride_w, cpad_w, cdil_w;
 };
 
 struct hrn_module {
@@ -322,9 +323,11 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
         if ((int64_t)p->m * p->lda * es >= (1ll << 31)) return fail(HRN_E_BADPARAM, "A operand exceeds 2 GiB per batch entry");
     } else {
         if (p->batch != 1) return fail(HRN_E_BADPARAM, "conv batch is the image count");
-        if (p->cstride < 1 || p->cdil < 1 || p->cpad < 0) return fail(HRN_E_BADPARAM, "conv stride/pad/dilation");
+        if (p->cstride < 1 || p->cdil < 1 || p->cpad < 0 || p->cstride_w < 1 || p->cdil_w < 1 || p->cpad_w < 0)
+            return fail(HRN_E_BADPARAM, "conv stride/pad/dilation (height %d/%d/%d, width %d/%d/%d)", p->cstride, p->cpad,
+                        p->cdil, p->cstride_w, p->cpad_w, p->cdil_w);
         const int ho = (p->ch - ((p->kh - 1) * p->cdil + 1) + 2 * p->cpad) / p->cstride + 1;
-        const int wo = (p->cw - ((p->kw - 1) * p->cdil + 1) + 2 * p->cpad) / p->cstride + 1;
+        const int wo = (p->cw - ((p->kw - 1) * p->cdil_w + 1) + 2 * p->cpad_w) / p->cstride_w + 1;
         if (ho <= 0 || wo <= 0) return fail(HRN_E_BADPARAM, "conv output is empty");
         if (p->m != p->cn * ho * wo || p->n != p->co || p->k != p->kh * p->kw * p->ci)
             return fail(HRN_E_BADPARAM, "conv GEMM view (m,n,k)=(%d,%d,%d) inconsistent with the image shape", p->m, p->n, p->k);
@@ -332,12 +335,13 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
         if ((int64_t)p->cn * p->ch * p->cw * p->ci * es >= (1ll << 31)) return fail(HRN_E_BADPARAM, "input exceeds 2 GiB");
         k->H = p->ch; k->W = p->cw; k->CI = p->ci; k->HO = ho; k->WO = wo; k->KH = p->kh; k->KW = p->kw;
         k->cstride = p->cstride; k->cpad = p->cpad; k->cdil = p->cdil;
+        k->cstride_w = p->cstride_w; k->cpad_w = p->cpad_w; k->cdil_w = p->cdil_w;
         if (d.conv_window) {
-            if (p->cstride != 1 || p->cdil != 1 || ho != p->ch || wo != p->cw)
+            if (p->cstride != 1 || p->cdil != 1 || p->cstride_w != 1 || p->cdil_w != 1 || ho != p->ch || wo != p->cw)
                 return fail(HRN_E_BADPARAM, "conv_window needs stride 1, dilation 1 and 'same' padding");
             if ((p->ci * es) % d.bkb) return fail(HRN_E_BADPARAM, "conv_window needs CI*%d to be a multiple of bkb %d", es, d.bkb);
             if (p->kh * p->kw > 32) return fail(HRN_E_BADPARAM, "conv_window supports at most 32 filter taps");
-            const int64_t rows = d.bm + 2 * (int64_t)p->cpad * (p->cw + 1);
+            const int64_t rows = d.bm + 2 * ((int64_t)p->cpad * p->cw + p->cpad_w);
             const int64_t instr = (rows * (p->ci * es / 16) + 63) / 64;
             const int64_t dyn = instr * 1024;
             if (dyn + mod->info.lds_bytes > 163840)
@@ -695,17 +699,23 @@ void hrn_problem_gemm(hrn_problem* p, int batch, int m, int n, int k) {
     p->group_m = 8;
 }
 
-void hrn_problem_conv2d(hrn_problem* p, int n, int h, int w, int ci, int co, int kh, int kw, int stride, int pad, int dil) {
+void hrn_problem_conv2d_hw(hrn_problem* p, int n, int h, int w, int ci, int co, int kh, int kw, int stride_h, int stride_w,
+                           int pad_h, int pad_w, int dil_h, int dil_w) {
     memset(p, 0, sizeof *p);
     p->op = HRN_OP_CONV2D;
     p->batch = 1;
     p->cn = n; p->ch = h; p->cw = w; p->ci = ci; p->co = co; p->kh = kh; p->kw = kw;
-    p->cstride = stride; p->cpad = pad; p->cdil = dil;
-    const int ho = (stride > 0) ? (h - ((kh - 1) * dil + 1) + 2 * pad) / stride + 1 : 0;
-    const int wo = (stride > 0) ? (w - ((kw - 1) * dil + 1) + 2 * pad) / stride + 1 : 0;
+    p->cstride = stride_h; p->cpad = pad_h; p->cdil = dil_h;
+    p->cstride_w = stride_w; p->cpad_w = pad_w; p->cdil_w = dil_w;
+    const int ho = (stride_h > 0) ? (h - ((kh - 1) * dil_h + 1) + 2 * pad_h) / stride_h + 1 : 0;
+    const int wo = (stride_w > 0) ? (w - ((kw - 1) * dil_w + 1) + 2 * pad_w) / stride_w + 1 : 0;
     p->m = n * ho * wo; p->n = co; p->k = kh * kw * ci;
     p->lda = ci; p->ldb = p->k; p->ldc = co;
     p->group_m = 8;
+}
+
+void hrn_problem_conv2d(hrn_problem* p, int n, int h, int w, int ci, int co, int kh, int kw, int stride, int pad, int dil) {
+    hrn_problem_conv2d_hw(p, n, h, w, ci, co, kh, kw, stride, stride, pad, pad, dil, dil);
 }
 
 }  // extern "C"

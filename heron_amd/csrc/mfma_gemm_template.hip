@@ -42,6 +42,7 @@ struct HrnKArgs {
     // conv
     int32_t H, W, CI, HO, WO, KH, KW, cstride, cpad, cdil;
     int32_t pf_sa, pf_sb;       // L2 prefetch: column-tiles / row-tiles of the block one XCD runs concurrently
+    int32_t cstride_w, cpad_w, cdil_w;   // conv: the width-direction values (cstride/cpad/cdil are the height ones)
 };
 #endif
 
@@ -77,7 +78,7 @@ constexpr int PF = HRN_PF;
 constexpr int LOADM = HRN_LOAD;
 // Conv window mode (HRN_OP=1, stride 1, dilation 1, 'same' padding): instead of fetching an im2col tile of A for every
 // filter tap, the workgroup loads ONCE the window of input pixels its BM output pixels can reach (a contiguous range
-// of BM + 2*pad*(W+1) pixels, all channels) and every tap reads its operand fragments from that window at a row offset
+// of BM + 2*(pad_h*W + pad_w) pixels, all channels) and every tap reads its operand fragments from that window at a row offset
 // of r*W + s pixels; taps that fall into the padding are masked to zero in registers.  Only B (the filter) streams
 // through the LDS stages.
 #ifndef HRN_CONVWIN
@@ -278,7 +279,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
             const bool ok = m < a.M;
             voffA[i] = (uint32_t)img * (uint32_t)(a.H * a.W * a.CI) * ES;
             iy0[i] = ok ? oy * a.cstride - a.cpad : -(1 << 28);
-            ix0[i] = ox * a.cstride - a.cpad;
+            ix0[i] = ox * a.cstride_w - a.cpad_w;
             m += NW * RPI;
             ox += NW * RPI;
             while (ox >= a.WO) { ox -= a.WO; if (++oy == a.HO) { oy = 0; ++img; } }
@@ -322,7 +323,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
                 offA[i] = v;
             }
         } else if constexpr (!CW) {
-            const int iyr = cr * a.cdil, ixs = cs * a.cdil;
+            const int iyr = cr * a.cdil, ixs = cs * a.cdil_w;
             const bool kvalid = live && cr < a.KH;
 #pragma unroll
             for (int i = 0; i < A_LPW; ++i) {
@@ -396,10 +397,10 @@ hrn_mfma_kernel(const HrnKArgs a) {
     const int w_cch = CW ? w_pitch / BKB : 1;            // k-tiles per tap
     uint32_t tapmask[CW ? TM : 1];                       // bit t: tap t of this lane's pixel i is inside the image
     if constexpr (CW) {
-        const int w_rows = BM + 2 * a.cpad * (a.W + 1);  // pixels the BM outputs can reach
+        const int w_rows = BM + 2 * (a.cpad * a.W + a.cpad_w);  // pixels the BM outputs can reach
         const int cpp = w_pitch / 16;                    // 16-byte chunks per pixel
         const int n_instr = (w_rows * cpp + 63) / 64;    // 1 KiB wave loads that cover the window
-        const int gp0 = m0 - a.cpad * (a.W + 1);         // input pixel index of window row 0
+        const int gp0 = m0 - (a.cpad * a.W + a.cpad_w);  // input pixel index of window row 0
         for (int q = wave; q < n_instr; q += NW) {
             const int L = q * 64 + lane;
             const int wrow = L / cpp, pos = L - wrow * cpp;
@@ -421,7 +422,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
             if (m < a.M) {
                 for (int r = 0; r < a.KH; ++r)
                     for (int s2 = 0; s2 < a.KW; ++s2) {
-                        const int iy = oy + r - a.cpad, ix = ox + s2 - a.cpad;
+                        const int iy = oy + r - a.cpad, ix = ox + s2 - a.cpad_w;
                         if ((unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W) bits |= 1u << (r * a.KW + s2);
                     }
             }

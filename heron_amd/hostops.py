@@ -53,9 +53,168 @@ def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8):
     if CI != CI2:
         raise ValueError("channel mismatch")
     p = B.conv2d_problem(N, H, W, CI, CO, KH, KW, stride, pad, dil, group_m)
-    ho = (H - ((KH - 1) * dil + 1) + 2 * pad) // stride + 1
-    wo = (W - ((KW - 1) * dil + 1) + 2 * pad) // stride + 1
+    (sh, sw), (ph, pw), (dh, dw) = B._pair(stride), B._pair(pad), B._pair(dil)
+    ho = (H - ((KH - 1) * dh + 1) + 2 * ph) // sh + 1
+    wo = (W - ((KW - 1) * dw + 1) + 2 * pw) // sw + 1
     if out is None:
         out = torch.empty((N, ho, wo, CO), dtype=torch.float16 if f16 else torch.int32, device=X.device)
     mod.launch(p, X.data_ptr(), Wt.data_ptr(), out.data_ptr(), _stream())
     return out
+
+
+# ----------------------------------------------------------------------------------------------
+# Operand adapters: the reference declares several operators as "injective pre-stage + matrix product"
+# (layout changes, padding, constant right-hand sides).  An adapter is that pre-stage: it maps the caller's
+# tensors, in the reference's layouts, to the template's operands (A (M,K) / B (N,K), or NHWC / KRSC) and
+# maps the result back.  They only move, pad or generate data; every multiply-accumulate is the kernel's.
+def _pad_last(t, to):
+    if t.shape[-1] == to:
+        return t.contiguous()
+    out = torch.zeros(t.shape[:-1] + (to,), dtype=t.dtype, device=t.device)
+    out[..., :t.shape[-1]] = t
+    return out
+
+
+def _prep_identity(info, A, Bm):
+    return A, Bm
+
+
+def _prep_gemv(info, A, b):
+    K = info['gemm_view']['K']
+    Bp = torch.zeros((info['gemm_view']['N'], K), dtype=b.dtype, device=b.device)
+    Bp[0, :b.shape[-1]] = b.reshape(-1)
+    return _pad_last(A, K), Bp
+
+
+def _prep_scan(info, A):
+    g = info['gemm_view']
+    n = torch.arange(g['N'], device=A.device).unsqueeze(1)
+    k = torch.arange(g['K'], device=A.device).unsqueeze(0)
+    T = (n > k).to(torch.float16 if info['kind'] == 'f16' else torch.int8)
+    T[:, A.shape[-1]:] = 0
+    return _pad_last(A, g['K']), T
+
+
+def _prep_mean(info, In):
+    g = info['gemm_view']
+    N, C, H, W = In.shape
+    A = In.permute(1, 0, 2, 3).reshape(C, N * H * W)
+    Bm = torch.zeros((g['N'], g['K']), dtype=In.dtype, device=In.device)
+    Bm[0, :N * H * W] = 1.0 / (N * H * W)
+    return _pad_last(A, g['K']), Bm
+
+
+def _prep_var(info, In, Mean):
+    d = In - Mean
+    return _prep_mean(info, d * d)
+
+
+def _cpad(info):
+    return info['conv']['CI']
+
+
+def _prep_c1d_nwc(info, X, F):            # (N,W,CI), (K,CI,CO)
+    Xk = _pad_last(X, _cpad(info)).unsqueeze(1)
+    Wk = _pad_last(F.permute(2, 0, 1), _cpad(info)).unsqueeze(1)
+    return Xk, Wk.contiguous()
+
+
+def _prep_c1d_ncw(info, X, F):            # (N,CI,W), (CO,CI,KW)
+    Xk = _pad_last(X.permute(0, 2, 1), _cpad(info)).unsqueeze(1)
+    Wk = _pad_last(F.permute(0, 2, 1), _cpad(info)).unsqueeze(1)
+    return Xk, Wk.contiguous()
+
+
+def _prep_c2d_nchw(info, X, F):           # (N,CI,H,W), (CO,CI,KH,KW)
+    return _pad_last(X.permute(0, 2, 3, 1), _cpad(info)), _pad_last(F.permute(0, 2, 3, 1), _cpad(info))
+
+
+def _prep_c2d_hwio(info, X, F):           # (N,H,W,CI), (KH,KW,CI,CO)
+    return _pad_last(X, _cpad(info)), _pad_last(F.permute(3, 0, 1, 2), _cpad(info))
+
+
+def _prep_c3d_ndhwc(info, X, F):          # (N,D,H,W,CI), (KD,KH,KW,CI,CO)
+    dp = info['depth']
+    N, D, H, W, CI = X.shape
+    KD, DO, sd, pd, dd = dp['KD'], dp['DO'], dp['stride'], dp['pad'], dp['dil']
+    cip = info['conv']['CI'] // KD
+    Xp = torch.zeros((N, D + 2 * pd, H, W, cip), dtype=X.dtype, device=X.device)
+    Xp[:, pd:pd + D, :, :, :CI] = X
+    # depth taps side by side on the channel axis: channel block kd of output slice z is input slice z*sd + kd*dd
+    cols = torch.stack([Xp[:, kd * dd: kd * dd + (DO - 1) * sd + 1: sd] for kd in range(KD)], dim=4)
+    Xk = cols.reshape(N * DO, H, W, KD * cip).contiguous()
+    Fp = _pad_last(F.permute(4, 1, 2, 0, 3), cip)                    # (CO,KH,KW,KD,cip)
+    return Xk, Fp.reshape(Fp.shape[0], Fp.shape[1], Fp.shape[2], KD * cip).contiguous()
+
+
+def _prep_c3d_ncdhw(info, X, F):          # (N,CI,D,H,W), (CO,CI,KD,KH,KW)
+    return _prep_c3d_ndhwc(info, X.permute(0, 2, 3, 4, 1), F.permute(2, 3, 4, 1, 0))
+
+
+def _prep_t2d_nchw(info, X, F):           # (N,CI,H,W), (CO,CI,KH,KW)
+    t = info['transposed']
+    c = info['conv']
+    N, CI, H, W = X.shape
+    s = t['stride']
+    top = (c['KH'] - 1) * t['dil'] - t['pad']
+    left = (c['KW'] - 1) * t['dil'] - t['pad']
+    Xe = torch.zeros((N, c['H'], c['W'], c['CI']), dtype=X.dtype, device=X.device)
+    Xe[:, top: top + (H - 1) * s + 1: s, left: left + (W - 1) * s + 1: s, :CI] = X.permute(0, 2, 3, 1)
+    return Xe, _pad_last(F.permute(0, 2, 3, 1), c['CI'])
+
+
+def _fin_identity(info, C):
+    return C
+
+
+def _fin_c1d_nwc(info, C):                # (N,1,WO,CO) -> (N,WO,CO)
+    return C.squeeze(1)
+
+
+def _fin_c1d_ncw(info, C):                # -> (N,CO,WO)
+    return C.squeeze(1).permute(0, 2, 1).contiguous()
+
+
+def _fin_nchw(info, C):                   # (N,HO,WO,CO) -> (N,CO,HO,WO)
+    return C.permute(0, 3, 1, 2).contiguous()
+
+
+def _fin_c3d_ndhwc(info, C):              # (N*DO,HO,WO,CO) -> (N,DO,HO,WO,CO)
+    dp = info['depth']
+    return C.reshape(dp['N'], dp['DO'], C.shape[1], C.shape[2], C.shape[3])
+
+
+def _fin_c3d_ncdhw(info, C):              # -> (N,CO,DO,HO,WO)
+    return _fin_c3d_ndhwc(info, C).permute(0, 4, 1, 2, 3).contiguous()
+
+
+ADAPTERS = {
+    'identity': (_prep_identity, _fin_identity),
+    'gemv': (_prep_gemv, _fin_identity),
+    'scan': (_prep_scan, _fin_identity),
+    'mean': (_prep_mean, _fin_identity),
+    'var': (_prep_var, _fin_identity),
+    'c1d_nwc': (_prep_c1d_nwc, _fin_c1d_nwc),
+    'c1d_ncw': (_prep_c1d_ncw, _fin_c1d_ncw),
+    'c2d_nchw': (_prep_c2d_nchw, _fin_nchw),
+    'c2d_hwio': (_prep_c2d_hwio, _fin_identity),
+    'c3d_ndhwc': (_prep_c3d_ndhwc, _fin_c3d_ndhwc),
+    'c3d_ncdhw': (_prep_c3d_ncdhw, _fin_c3d_ncdhw),
+    't2d_nchw': (_prep_t2d_nchw, _fin_nchw),
+}
+
+
+def run_operator(mod, info, inputs, group_m=8):
+    """Runs one operator of the registry on device tensors given in the reference's own layouts.
+
+    ``info`` is the dictionary the operator definition handed to ``ctx.set_info``; ``mod`` an instance of the
+    template that matches its kind and operator."""
+    prep, fin = ADAPTERS[info.get('adapter', 'identity')]
+    A, Bm = prep(info, *inputs)
+    if info['operator'] == 'conv2d_nhwc':
+        c = info['conv']
+        C = conv2d_nhwc(mod, A, Bm, (c['stride'], c['stride_w']), (c['pad'], c['pad_w']), (c['dil'], c['dil_w']),
+                        group_m=group_m)
+    else:
+        C = gemm(mod, A, Bm, group_m=group_m)
+    return fin(info, C)

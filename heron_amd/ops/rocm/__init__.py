@@ -6,13 +6,27 @@ a config JSON to an operator definition ``opfunc(ctx, *shape, in_dtype, out_dtyp
 from .dense import heron_dense
 from .batch_matmul import heron_batch_matmul
 from .conv2d import heron_conv2d_nhwc
+from .conv_variants import (heron_conv1d_ncw, heron_conv1d_nwc, heron_conv2d_nchw, heron_conv2d_nchw_transposed,
+                            heron_conv3d_ncdhw, heron_conv3d_ndhwc, heron_dil_nhwc)
+from .reductions import heron_gemv, heron_mean, heron_scan, heron_var
 
 
 def getOpFromName(name):
     opmap = {
         "gemm": heron_dense,
         "bmm": heron_batch_matmul,
-        "c2d": heron_conv2d_nhwc,
+        "c2d": heron_conv2d_nhwc,                 # NHWC, as ops/x86 and the benchmark configs; NCHW is "c2d_nchw"
         "c2d_nhwc": heron_conv2d_nhwc,
+        "c2d_nchw": heron_conv2d_nchw,
+        "gemv": heron_gemv,
+        "scan": heron_scan,
+        "mean": heron_mean,
+        "var": heron_var,
+        "c1d": heron_conv1d_ncw,
+        "c1d_nwc": heron_conv1d_nwc,
+        "c3d": heron_conv3d_ncdhw,
+        "c3d_ndhwc": heron_conv3d_ndhwc,
+        "dil": heron_dil_nhwc,
+        "t2d": heron_conv2d_nchw_transposed,
     }
     return opmap[name]

@@ -17,6 +17,11 @@ from ..tensor import compute, placeholder
 from .common import element_kind, mfma_info
 
 
+def pair(v):
+    """int or (height, width) pair, as the reference's operators accept (ops/cuda/conv2d.py:143-153)."""
+    return (int(v), int(v)) if isinstance(v, int) else (int(v[0]), int(v[1]))
+
+
 def conv_out_size(size, k, stride, pad, dil):
     return (size - ((k - 1) * dil + 1) + 2 * pad) // stride + 1
 
@@ -27,8 +32,7 @@ W_FORMATS = ("OhwI64o4i", "OhwI48o4i", "OhwI32o4i")
 def heron_conv2d_nhwc(ctx, N, H, W, CI, CO, KH, KW, stride, padding, dilation, *dtypes):
     """``dtypes`` is (in_dtype, out_dtype) as in ops/cuda/conv2d.py:137-141, or (w_format, in_dtype, out_dtype)
     as in ops/x86/conv2d_int8.py:31-35."""
-    assert isinstance(stride, int) and isinstance(padding, int) and isinstance(dilation, int), \
-        "square stride/padding/dilation"
+    (sh, sw), (ph, pw), (dh, dw) = pair(stride), pair(padding), pair(dilation)
     w_format = None
     if len(dtypes) == 3:
         w_format, in_dtype, out_dtype = dtypes
@@ -42,13 +46,14 @@ def heron_conv2d_nhwc(ctx, N, H, W, CI, CO, KH, KW, stride, padding, dilation, *
         raise ValueError("w_format belongs to the quantized operator")
     if kind == "f16" and CI % 8 or kind == "u8s8" and CI % 16:
         raise ValueError("CI must cover whole 16-byte channel chunks (multiple of 8 for fp16, 16 for uint8)")
-    HO = conv_out_size(H, KH, stride, padding, dilation)
-    WO = conv_out_size(W, KW, stride, padding, dilation)
+    HO = conv_out_size(H, KH, sh, ph, dh)
+    WO = conv_out_size(W, KW, sw, pw, dw)
     a_dt, b_dt, o_dt = ("float16", "float16", "float16") if kind == "f16" else ("uint8", "int8", "int32")
     Input = placeholder((N, H, W, CI), "input", a_dt)
     Filter = placeholder((CO, KH, KW, CI), "filter", b_dt)
     out = compute((N, HO, WO, CO), "out", o_dt, [Input, Filter], tag="conv2d_nhwc_mfma")
-    conv = dict(w_format=w_format, N=N, H=H, W=W, CI=CI, CO=CO, KH=KH, KW=KW, stride=stride, pad=padding, dil=dilation, HO=HO, WO=WO)
+    conv = dict(w_format=w_format, N=N, H=H, W=W, CI=CI, CO=CO, KH=KH, KW=KW, stride=sh, pad=ph, dil=dh, stride_w=sw, pad_w=pw, dil_w=dw,
+                HO=HO, WO=WO)
     ctx.set_info(mfma_info(kind, out.op.name, Input.name, Filter.name,
                            dict(batch=1, M=N * HO * WO, N=CO, K=KH * KW * CI), 'conv2d_nhwc', {'conv': conv}))
     ctx.set_axis_map({

@@ -29,7 +29,7 @@ _spawn = mp.get_context("spawn")
 
 
 def _problem_to_dict(p):
-    return {name: (list(getattr(p, name)) if name == "reserved" else int(getattr(p, name))) for name, _ in p._fields_}
+    return {name: int(getattr(p, name)) for name, _ in p._fields_}
 
 
 def _compile_worker(desc_tuple, timeout_s):
@@ -141,8 +141,7 @@ def _server_main(conn, device_id):
             mod = mods[desc_tuple]
             p = B.Problem()
             for k, v in prob.items():
-                if k != "reserved":
-                    setattr(p, k, v)
+                setattr(p, k, v)
             tensors = []
             for i, (shape, dtype) in enumerate(arg_info):
                 tdt = getattr(torch, _TORCH_DT[dtype])

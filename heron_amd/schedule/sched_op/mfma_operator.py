@@ -38,8 +38,9 @@ class TemplateSchedule:
         g = self.info['gemm_view']
         if self.info['operator'] == 'conv2d_nhwc':
             c = self.info['conv']
-            return B.conv2d_problem(c['N'], c['H'], c['W'], c['CI'], c['CO'], c['KH'], c['KW'], c['stride'],
-                                    c['pad'], c['dil'], self.params['group_m'])
+            return B.conv2d_problem(c['N'], c['H'], c['W'], c['CI'], c['CO'], c['KH'], c['KW'],
+                                    (c['stride'], c['stride_w']), (c['pad'], c['pad_w']), (c['dil'], c['dil_w']),
+                                    self.params['group_m'])
         return B.gemm_problem(g['batch'], g['M'], g['N'], g['K'], self.params['group_m'])
 
     def describe(self):
@@ -194,9 +195,10 @@ class convWindowOp(schedOp):
         halo = 0
         if s.info['operator'] == 'conv2d_nhwc':
             c = s.info['conv']
-            ok = (c['stride'] == 1 and c['dil'] == 1 and c['HO'] == c['H'] and c['WO'] == c['W'] and c['KH'] * c['KW'] <= 32)
+            ok = (c['stride'] == 1 and c['dil'] == 1 and c['stride_w'] == 1 and c['dil_w'] == 1 and
+                  c['HO'] == c['H'] and c['WO'] == c['W'] and c['KH'] * c['KW'] <= 32)
             pitch = c['CI'] * (2 if s.info['kind'] == 'f16' else 1)
-            halo = 2 * c['pad'] * (c['W'] + 1)
+            halo = 2 * (c['pad'] * c['W'] + c['pad_w'])
         win = self.knob(ctx, stage_name, 'conv_window', [0, 1] if ok else [0], 1 if ok else 0)
         staged = self.var(ctx, stage_name, 'a_rows_staged', 0, 512, 16)       # rows of A that go through the stages
         off = self.var(ctx, stage_name, 'conv_window_off', 0, 1, 1)

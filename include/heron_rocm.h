@@ -107,11 +107,12 @@ typedef struct hrn_problem {
     int32_t m, n, k;
     int32_t lda, ldb, ldc;
     int64_t stride_a, stride_b, stride_c;
-    /* conv only */
+    /* conv only; cstride/cpad/cdil act on the height, the *_w fields on the width (the reference's operators take
+     * an int or an (h, w) pair for each, ops/cuda/conv2d.py:143-153); padding is symmetric per direction */
     int32_t cn, ch, cw, ci, co, kh, kw, cstride, cpad, cdil;
     /* launch-time raster knob: tiles are walked in column groups of this many row-tiles */
     int32_t group_m;
-    int32_t reserved[3];
+    int32_t cstride_w, cpad_w, cdil_w;
 } hrn_problem;
 
 typedef struct hrn_module hrn_module;
@@ -193,6 +194,8 @@ int hrn_probe_copy(const void* src, void* dst, size_t bytes, int repeat, double*
 void hrn_problem_gemm(hrn_problem* p, int batch, int m, int n, int k);
 void hrn_problem_conv2d(hrn_problem* p, int n, int h, int w, int ci, int co, int kh, int kw,
                         int stride, int pad, int dil);
+void hrn_problem_conv2d_hw(hrn_problem* p, int n, int h, int w, int ci, int co, int kh, int kw,
+                           int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w);
 
 const char* hrn_last_error(void);
 const char* hrn_version(void);

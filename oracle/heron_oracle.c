@@ -223,13 +223,15 @@ ORC_API void orc_bmm_f32(const float* A, const float* B, float* C,
 /*
  * ops/cuda/conv2d.py:166-196.  In (N,H,W,CI), Wt (CO,KH,KW,CI), Out (N,HO,WO,CO),
  * HO = (H - ((KH-1)*dil+1) + 2*pad)/stride + 1 (conv2d.py:168-175); taps that fall into
- * the zero padding contribute nothing.
+ * the zero padding contribute nothing.  stride/pad/dil act on the height, the *_w values on the width
+ * (conv2d.py:143-153 accepts an int or a pair for each).
  */
 ORC_API void orc_conv2d_nhwc_f32(const float* In, const float* Wt, float* Out,
                                  int64_t N, int64_t H, int64_t W, int64_t CI, int64_t CO,
-                                 int64_t KH, int64_t KW, int64_t stride, int64_t pad, int64_t dil) {
+                                 int64_t KH, int64_t KW, int64_t stride, int64_t stride_w, int64_t pad, int64_t pad_w,
+                                     int64_t dil, int64_t dil_w) {
     const int64_t HO = (H - ((KH - 1) * dil + 1) + 2 * pad) / stride + 1;
-    const int64_t WO = (W - ((KW - 1) * dil + 1) + 2 * pad) / stride + 1;
+    const int64_t WO = (W - ((KW - 1) * dil_w + 1) + 2 * pad_w) / stride_w + 1;
 #pragma omp parallel for collapse(3) schedule(static)
     for (int64_t n = 0; n < N; ++n)
         for (int64_t y = 0; y < HO; ++y)
@@ -240,7 +242,7 @@ ORC_API void orc_conv2d_nhwc_f32(const float* In, const float* Wt, float* Out,
                         const int64_t iy = y * stride + ry * dil - pad;
                         if (iy < 0 || iy >= H) continue;
                         for (int64_t rx = 0; rx < KW; ++rx) {
-                            const int64_t ix = x * stride + rx * dil - pad;
+                            const int64_t ix = x * stride_w + rx * dil_w - pad_w;
                             if (ix < 0 || ix >= W) continue;
                             const float* a = In + ((n * H + iy) * W + ix) * CI;
                             const float* w = Wt + ((f * KH + ry) * KW + rx) * CI;
@@ -257,9 +259,10 @@ ORC_API void orc_conv2d_nhwc_f32(const float* In, const float* Wt, float* Out,
  */
 ORC_API void orc_conv2d_nhwc_u8s8s32(const uint8_t* In, const int8_t* Wt, int32_t* Out,
                                      int64_t N, int64_t H, int64_t W, int64_t CI, int64_t CO,
-                                     int64_t KH, int64_t KW, int64_t stride, int64_t pad, int64_t dil) {
+                                     int64_t KH, int64_t KW, int64_t stride, int64_t stride_w, int64_t pad, int64_t pad_w,
+                                     int64_t dil, int64_t dil_w) {
     const int64_t HO = (H - ((KH - 1) * dil + 1) + 2 * pad) / stride + 1;
-    const int64_t WO = (W - ((KW - 1) * dil + 1) + 2 * pad) / stride + 1;
+    const int64_t WO = (W - ((KW - 1) * dil_w + 1) + 2 * pad_w) / stride_w + 1;
 #pragma omp parallel for collapse(3) schedule(static)
     for (int64_t n = 0; n < N; ++n)
         for (int64_t y = 0; y < HO; ++y)
@@ -270,7 +273,7 @@ ORC_API void orc_conv2d_nhwc_u8s8s32(const uint8_t* In, const int8_t* Wt, int32_
                         const int64_t iy = y * stride + ry * dil - pad;
                         if (iy < 0 || iy >= H) continue;
                         for (int64_t rx = 0; rx < KW; ++rx) {
-                            const int64_t ix = x * stride + rx * dil - pad;
+                            const int64_t ix = x * stride_w + rx * dil_w - pad_w;
                             if (ix < 0 || ix >= W) continue;
                             const uint8_t* a = In + ((n * H + iy) * W + ix) * CI;
                             const int8_t* w = Wt + ((f * KH + ry) * KW + rx) * CI;

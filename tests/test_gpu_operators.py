@@ -1,0 +1,165 @@
+"""GPU parity of the operators declared as "pre-stage + product" (gemv, scan, mean, var, conv1d/2d/3d layouts,
+dilated and transposed conv): operands in the reference's layouts go through the operand adapter and the MFMA
+template, the result is compared with the float64 / int64 restatement of the reference declaration.
+
+fp16: max|err| / max|ref| <= 1e-2 (fp16 inputs, fp32 accumulate, one rounding); integer forms bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from heron_amd import backend as B
+from heron_amd import hostops, instances
+from heron_amd.ops.rocm import getOpFromName
+
+pytestmark = pytest.mark.gpu
+REL_TOL = 1e-2
+_mods = {}
+
+
+class Ctx:
+    def set_info(self, info):
+        self.info = info
+
+    def set_axis_map(self, m):
+        self.axis_map = m
+
+
+def declare(name, args, dtype):
+    c = Ctx()
+    out = getOpFromName(name)(c, *args, dtype, dtype)
+    return c.info, out[0]
+
+
+def module(info):
+    f16 = info['kind'] == 'f16'
+    if info['operator'] == 'conv2d_nhwc':
+        d = instances.D(instances.F16, instances.CONV, *instances.PARITY_SHAPES[4]) if f16 else instances.int8_conv_descs()[0]
+    else:
+        d = instances.BEST["small_f16"] if f16 else instances.BEST["small"]
+    key = d.as_tuple()
+    if key not in _mods:
+        _mods[key] = B.Module(d)
+    return _mods[key]
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def rnd(shape, seed, dtype):
+    rng = np.random.default_rng(seed)
+    if dtype == "float16":
+        return rng.normal(0, 1, shape).astype(np.float16)
+    if dtype == "uint8":
+        return rng.integers(0, 256, shape, dtype=np.uint8)
+    return rng.integers(-128, 128, shape, dtype=np.int8)
+
+
+def check(got, ref, f16):
+    got = got.cpu().numpy()
+    assert got.shape == ref.shape, (got.shape, ref.shape)
+    if f16:
+        scale = float(np.abs(ref).max()) + 1e-30
+        assert float(np.abs(got.astype(np.float64) - ref).max()) / scale <= REL_TOL
+    else:
+        assert got.dtype == np.int32 and np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+def test_gemv_and_scan(dtype, hrn):
+    f16 = dtype == "float16"
+    a_dt, b_dt = ("float16", "float16") if f16 else ("uint8", "int8")
+    for M, K in [(100, 72), (513, 1000), (64, 4096)]:
+        info, out = declare("gemv", [M, K], dtype)
+        A, b = rnd((M, K), 1, a_dt), rnd((1, K), 2, b_dt)
+        print("gemv", dtype, M, K, flush=True)
+        check(hostops.run_operator(module(info), info, [dev(A), dev(b)]), oracle.gemv_ref(A, b), f16)
+    for M, N, K in [(64, 128, 128), (50, 40, 200), (7, 300, 104)]:
+        info, out = declare("scan", [M, N, K], dtype)
+        A = rnd((M, K), 3, a_dt)
+        print("scan", dtype, M, N, K, flush=True)
+        check(hostops.run_operator(module(info), info, [dev(A)]), oracle.scan_ref(A, N), f16)
+
+
+def test_mean_and_var(hrn):
+    for shape in [(4, 64, 14, 14), (3, 20, 7, 9), (1, 128, 28, 28)]:
+        info, out = declare("mean", list(shape), "float16")
+        In = rnd(shape, 4, "float16")
+        print("mean/var", shape, flush=True)
+        check(hostops.run_operator(module(info), info, [dev(In)]), oracle.mean_ref(In), True)
+        Mean = np.broadcast_to(In.astype(np.float64).mean(axis=(0, 2, 3), keepdims=True), shape).astype(np.float16)
+        info, out = declare("var", list(shape), "float16")
+        check(hostops.run_operator(module(info), info, [dev(In), dev(Mean)]), oracle.var_ref(In, Mean), True)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+def test_conv1d_layouts(dtype, hrn):
+    f16 = dtype == "float16"
+    a_dt, b_dt = ("float16", "float16") if f16 else ("uint8", "int8")
+    for (N, W, CI, CO, K, s, p, d) in [(8, 100, 16, 32, 3, 1, 1, 1), (3, 57, 24, 20, 5, 2, 2, 1), (2, 64, 48, 8, 3, 1, 2, 2)]:
+        X, F = rnd((N, W, CI), 5, a_dt), rnd((K, CI, CO), 6, b_dt)
+        print("c1d", dtype, (N, W, CI, CO, K, s, p, d), flush=True)
+        info, _ = declare("c1d_nwc", [N, W, CI, CO, K, s, p, d], dtype)
+        check(hostops.run_operator(module(info), info, [dev(X), dev(F)]), oracle.conv1d_nwc_ref(X, F, s, p, d), f16)
+        if d == 1:                                   # the NCW declaration asserts dilation == 1 (conv1d.py:17)
+            info, _ = declare("c1d", [N, W, CI, CO, K, s, p, d], dtype)
+            Xc, Fc = X.transpose(0, 2, 1), F.transpose(2, 1, 0)
+            check(hostops.run_operator(module(info), info, [dev(Xc), dev(Fc)]), oracle.conv1d_ncw_ref(Xc, Fc, s, p, d), f16)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+def test_conv2d_nchw_dilated_and_transposed(dtype, hrn):
+    f16 = dtype == "float16"
+    a_dt, b_dt = ("float16", "float16") if f16 else ("uint8", "int8")
+    # first-layer shape with CI = 3 (channel padding), (h, w) pairs, plain
+    for (N, H, W, CI, CO, KH, KW, s, p, d) in [(2, 20, 20, 3, 16, 7, 7, 2, 3, 1), (1, 12, 15, 16, 24, 3, 5, (2, 1), (1, 2), 1),
+                                               (2, 9, 9, 32, 8, 3, 3, 1, 1, 1)]:
+        X, F = rnd((N, CI, H, W), 7, a_dt), rnd((CO, CI, KH, KW), 8, b_dt)
+        print("c2d_nchw", dtype, (N, H, W, CI, CO, KH, KW, s, p, d), flush=True)
+        info, _ = declare("c2d_nchw", [N, H, W, CI, CO, KH, KW, s, p, d], dtype)
+        check(hostops.run_operator(module(info), info, [dev(X), dev(F)]), oracle.conv2d_nchw_ref(X, F, s, p, d), f16)
+    for (N, H, W, CI, CO, KH, KW, s, p, d) in [(2, 20, 20, 16, 16, 3, 3, 1, 2, 2), (1, 17, 13, 8, 12, 3, 3, 2, 3, 3)]:
+        X, F = rnd((N, H, W, CI), 9, a_dt), rnd((KH, KW, CI, CO), 10, b_dt)
+        print("dil", dtype, (N, H, W, CI, CO, KH, KW, s, p, d), flush=True)
+        info, _ = declare("dil", [N, H, W, CI, CO, KH, KW, s, p, d], dtype)
+        check(hostops.run_operator(module(info), info, [dev(X), dev(F)]), oracle.dil_nhwc_ref(X, F, s, p, d), f16)
+    for (N, H, W, CI, CO, KH, KW, s, p, d, op) in [(2, 7, 7, 16, 8, 4, 4, 2, 1, 1, 0), (1, 5, 6, 8, 12, 3, 3, 2, 1, 1, 1),
+                                                   (2, 6, 5, 16, 4, 3, 3, 1, 0, 1, 0), (1, 4, 4, 16, 8, 3, 3, 3, 2, 2, 1)]:
+        X, F = rnd((N, CI, H, W), 11, a_dt), rnd((CO, CI, KH, KW), 12, b_dt)
+        print("t2d", dtype, (N, H, W, CI, CO, KH, KW, s, p, d, op), flush=True)
+        info, _ = declare("t2d", [N, H, W, CI, CO, KH, KW, s, p, d, op], dtype)
+        check(hostops.run_operator(module(info), info, [dev(X), dev(F)]),
+              oracle.conv2d_transposed_nchw_ref(X, F, s, p, d, op), f16)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+def test_conv3d_layouts(dtype, hrn):
+    f16 = dtype == "float16"
+    a_dt, b_dt = ("float16", "float16") if f16 else ("uint8", "int8")
+    for (N, D, H, W, CI, CO, KD, KH, KW, s, p, d) in [(2, 8, 10, 10, 16, 16, 3, 3, 3, 1, 1, 1),
+                                                      (1, 6, 9, 7, 8, 12, 3, 3, 2, (2, 1, 1), (1, 1, 0), 1),
+                                                      (1, 7, 8, 8, 16, 8, 2, 3, 3, 1, (0, 2, 1), (2, 2, 1))]:
+        X, F = rnd((N, D, H, W, CI), 13, a_dt), rnd((KD, KH, KW, CI, CO), 14, b_dt)
+        print("c3d", dtype, (N, D, H, W, CI, CO, KD, KH, KW, s, p, d), flush=True)
+        info, _ = declare("c3d_ndhwc", [N, D, H, W, CI, CO, KD, KH, KW, s, p, d], dtype)
+        check(hostops.run_operator(module(info), info, [dev(X), dev(F)]), oracle.conv3d_ndhwc_ref(X, F, s, p, d), f16)
+        if d == 1:                                   # the NCDHW declaration asserts dilation == 1 (conv3d.py:15)
+            Xc, Fc = X.transpose(0, 4, 1, 2, 3), F.transpose(4, 3, 0, 1, 2)
+            info, _ = declare("c3d", [N, D, H, W, CI, CO, KD, KH, KW, s, p, d], dtype)
+            check(hostops.run_operator(module(info), info, [dev(Xc), dev(Fc)]), oracle.conv3d_ncdhw_ref(Xc, Fc, s, p, d), f16)
+
+
+def test_conv2d_nhwc_height_width_pairs(hrn):
+    """(h, w) stride / padding / dilation pairs on the native NHWC operator, both element kinds."""
+    for dtype in ("float16", "int8"):
+        f16 = dtype == "float16"
+        a_dt, b_dt = ("float16", "float16") if f16 else ("uint8", "int8")
+        for (N, H, W, CI, CO, KH, KW, s, p, d) in [(1, 9, 12, 16, 16, 3, 2, (2, 1), (1, 0), (1, 2)), (2, 1, 33, 32, 8, 1, 3, (1, 2), (0, 2), 1),
+                                                   (1, 10, 7, 16, 4, 2, 3, 1, (0, 1), (3, 1))]:
+            X, Wt = rnd((N, H, W, CI), 15, a_dt), rnd((CO, KH, KW, CI), 16, b_dt)
+            print("c2d pairs", dtype, (N, H, W, CI, CO, KH, KW, s, p, d), flush=True)
+            info, _ = declare("c2d", [N, H, W, CI, CO, KH, KW, s, p, d], dtype)
+            ref = oracle.conv2d_nhwc_f32(X, Wt, s, p, d).astype(np.float64) if f16 else oracle.conv2d_nhwc_u8s8s32(X, Wt, s, p, d)
+            check(hostops.run_operator(module(info), info, [dev(X), dev(Wt)]), ref, f16)

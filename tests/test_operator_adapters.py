@@ -1,0 +1,90 @@
+"""Operand adapters on the CPU: pre-stage -> (oracle product in place of the kernel) -> post-stage must equal the
+restatement of the reference declaration.  This checks the layout/padding logic of ``hostops.ADAPTERS`` and the
+GEMM / conv views the operator definitions announce, without a GPU; the kernel itself is covered by the GPU tests.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from heron_amd import hostops
+from heron_amd.ops.rocm import getOpFromName
+
+
+class Ctx:
+    def set_info(self, info):
+        self.info = info
+
+    def set_axis_map(self, m):
+        self.axis_map = m
+
+
+def rnd(shape, seed):
+    return np.random.default_rng(seed).normal(0, 1, shape).astype(np.float16)
+
+
+def through_adapter(name, args, inputs):
+    c = Ctx()
+    out = getOpFromName(name)(c, *args, "float16", "float16")
+    info = c.info
+    prep, fin = hostops.ADAPTERS[info['adapter']]
+    A, Bm = prep(info, *[torch.from_numpy(np.ascontiguousarray(x)) for x in inputs])
+    g = info['gemm_view']
+    if info['operator'] == 'conv2d_nhwc':
+        cv = info['conv']
+        assert tuple(A.shape) == (cv['N'], cv['H'], cv['W'], cv['CI']) and tuple(Bm.shape) == (cv['CO'], cv['KH'], cv['KW'], cv['CI'])
+        C = oracle.conv2d_nhwc_f32(A.numpy(), Bm.numpy(), (cv['stride'], cv['stride_w']), (cv['pad'], cv['pad_w']),
+                                   (cv['dil'], cv['dil_w']))
+        assert C.shape == out[0].shape and C.shape[0] * C.shape[1] * C.shape[2] == g['M']
+    else:
+        assert tuple(A.shape) == (g['M'], g['K']) and tuple(Bm.shape) == (g['N'], g['K'])
+        C = oracle.gemm_f32(A.numpy(), Bm.numpy())
+    assert A.is_contiguous() and Bm.is_contiguous()
+    return fin(info, torch.from_numpy(C)).numpy()
+
+
+def close(got, ref):
+    assert got.shape == ref.shape
+    assert np.abs(got - ref).max() <= 1e-4 * (np.abs(ref).max() + 1)
+
+
+def test_reductions():
+    A, b = rnd((33, 100), 1), rnd((1, 100), 2)
+    close(through_adapter("gemv", [33, 100], [A, b]), oracle.gemv_ref(A, b))
+    close(through_adapter("scan", [33, 40, 100], [A]), oracle.scan_ref(A, 40))
+    In = rnd((3, 20, 7, 9), 3)
+    close(through_adapter("mean", [3, 20, 7, 9], [In]), oracle.mean_ref(In))
+    Mean = np.broadcast_to(In.astype(np.float64).mean(axis=(0, 2, 3), keepdims=True), In.shape).astype(np.float16)
+    close(through_adapter("var", [3, 20, 7, 9], [In, Mean]), oracle.var_ref(In, Mean))
+
+
+@pytest.mark.parametrize("s,p,d", [(1, 1, 1), (2, 2, 1), (1, 2, 2)])
+def test_conv1d(s, p, d):
+    X, F = rnd((3, 57, 12), 4), rnd((5, 12, 20), 5)
+    close(through_adapter("c1d_nwc", [3, 57, 12, 20, 5, s, p, d], [X, F]), oracle.conv1d_nwc_ref(X, F, s, p, d))
+    Xc, Fc = X.transpose(0, 2, 1), F.transpose(2, 1, 0)
+    close(through_adapter("c1d", [3, 57, 12, 20, 5, s, p, d], [Xc, Fc]), oracle.conv1d_ncw_ref(Xc, Fc, s, p, d))
+
+
+def test_conv2d_variants():
+    X, F = rnd((2, 3, 20, 20), 6), rnd((16, 3, 7, 7), 7)
+    close(through_adapter("c2d_nchw", [2, 20, 20, 3, 16, 7, 7, 2, 3, 1], [X, F]), oracle.conv2d_nchw_ref(X, F, 2, 3, 1))
+    X, F = rnd((1, 16, 12, 15), 8), rnd((24, 16, 3, 5), 9)
+    close(through_adapter("c2d_nchw", [1, 12, 15, 16, 24, 3, 5, (2, 1), (1, 2), 1], [X, F]),
+          oracle.conv2d_nchw_ref(X, F, (2, 1), (1, 2), 1))
+    X, F = rnd((1, 17, 13, 8), 10), rnd((3, 3, 8, 12), 11)
+    close(through_adapter("dil", [1, 17, 13, 8, 12, 3, 3, 2, 3, 3], [X, F]), oracle.dil_nhwc_ref(X, F, 2, 3, 3))
+
+
+@pytest.mark.parametrize("s,p,d,op", [(2, 1, 1, 0), (2, 1, 1, 1), (1, 0, 1, 0), (3, 2, 2, 1)])
+def test_conv2d_transposed(s, p, d, op):
+    X, F = rnd((2, 6, 5, 6), 12), rnd((4, 6, 3, 4), 13)
+    close(through_adapter("t2d", [2, 5, 6, 6, 4, 3, 4, s, p, d, op], [X, F]), oracle.conv2d_transposed_nchw_ref(X, F, s, p, d, op))
+
+
+@pytest.mark.parametrize("s,p,d", [(1, 1, 1), ((2, 1, 1), (1, 1, 0), 1), (1, (0, 2, 1), (2, 2, 1))])
+def test_conv3d(s, p, d):
+    X, F = rnd((2, 6, 9, 7, 5), 14), rnd((3, 3, 2, 5, 12), 15)
+    close(through_adapter("c3d_ndhwc", [2, 6, 9, 7, 5, 12, 3, 3, 2, s, p, d], [X, F]), oracle.conv3d_ndhwc_ref(X, F, s, p, d))
+    Xc, Fc = X.transpose(0, 4, 1, 2, 3), F.transpose(4, 3, 0, 1, 2)
+    close(through_adapter("c3d", [2, 6, 9, 7, 5, 12, 3, 3, 2, s, p, d], [Xc, Fc]), oracle.conv3d_ncdhw_ref(Xc, Fc, s, p, d))

@@ -110,6 +110,24 @@ def test_conv_against_torch_library_routine(case):
     assert np.abs(got - ref).max() <= 1e-5 * (np.abs(ref).max() + 1)
 
 
+@pytest.mark.parametrize("case", [(1, 9, 12, 4, 3, 3, 2, (2, 1), (1, 0), (1, 2)), (2, 1, 17, 8, 5, 1, 3, (1, 2), (0, 2), (1, 1)),
+                                  (1, 10, 7, 2, 2, 2, 3, (1, 1), (0, 1), (3, 1))])
+def test_conv_height_and_width_parameters_differ(case):
+    """stride/padding/dilation given as (height, width) pairs, fp32 and integer forms, against torch."""
+    N, H, W, CI, CO, KH, KW, s, p, d = case
+    X, Wt = workloads.conv2d_inputs(N, H, W, CI, CO, KH, KW, seed=3)
+    x = torch.from_numpy(X.astype(np.float64)).permute(0, 3, 1, 2)
+    w = torch.from_numpy(Wt.astype(np.float64)).permute(0, 3, 1, 2)
+    ref = torch.nn.functional.conv2d(x, w, stride=s, padding=p, dilation=d).permute(0, 2, 3, 1).numpy()
+    got = oracle.conv2d_nhwc_f32(X, Wt, s, p, d)
+    assert got.shape == ref.shape and np.abs(got - ref).max() <= 1e-5 * (np.abs(ref).max() + 1)
+    Xi, Wi = workloads.conv2d_u8s8_inputs(N, H, W, CI, CO, KH, KW, seed=4)
+    xi = torch.from_numpy(Xi.astype(np.float64)).permute(0, 3, 1, 2)
+    wi = torch.from_numpy(Wi.astype(np.float64)).permute(0, 3, 1, 2)
+    refi = torch.nn.functional.conv2d(xi, wi, stride=s, padding=p, dilation=d).permute(0, 2, 3, 1).numpy()
+    assert np.array_equal(oracle.conv2d_nhwc_u8s8s32(Xi, Wi, s, p, d), refi.astype(np.int64))
+
+
 def test_conv_1x1_reduces_to_gemm():
     X, Wt = workloads.conv2d_inputs(2, 5, 6, 8, 7, 1, 1, seed=9)
     got = oracle.conv2d_nhwc_f32(X, Wt)
@@ -196,3 +214,69 @@ def test_workload_generators_are_seeded_and_shaped():
     assert 0.3 < (X == 0).mean() < 0.7
     assert workloads.gemm_work(8192, 8192, 8192, 1, 4) == (2 * 8192 ** 3, 402653184)
     assert workloads.conv_work(32, 56, 56, 64, 64, 3, 3, 1, 1, 1) == (7398752256, 25763840)
+
+
+# ---------------------------------------------------------------- operators built on a pre-stage + product
+def _rand(shape, seed, scale=1.0):
+    return (np.random.default_rng(seed).normal(0, scale, shape)).astype(np.float16)
+
+
+def test_gemv_scan_mean_var_against_numpy_routines():
+    A, b = _rand((7, 24), 1), _rand((1, 24), 2)
+    g = oracle.gemv_ref(A, b)
+    assert g.shape == (7, 8) and np.allclose(g[:, 0], A.astype(np.float64) @ b.astype(np.float64)[0]) and not g[:, 1:].any()
+    s = oracle.scan_ref(A, 24)
+    excl = np.cumsum(A.astype(np.float64), axis=1) - A.astype(np.float64)           # exclusive prefix sum
+    assert np.allclose(s, excl)
+    Ai = np.random.default_rng(3).integers(0, 256, (5, 32), dtype=np.uint8)
+    assert np.array_equal(oracle.scan_ref(Ai, 32), np.cumsum(Ai.astype(np.int64), 1) - Ai)
+    In = _rand((3, 5, 4, 6), 4)
+    m = oracle.mean_ref(In)
+    assert m.shape == (5, 8) and not m[:, 1:].any()
+    assert np.allclose(m[:, 0], In.astype(np.float64).mean(axis=(0, 2, 3)), rtol=1e-3)   # 1/72 rounded to fp16
+    Mean = np.broadcast_to(In.astype(np.float64).mean(axis=(0, 2, 3), keepdims=True), In.shape).astype(np.float16)
+    v = oracle.var_ref(In, Mean)
+    assert np.allclose(v[:, 0], In.astype(np.float64).var(axis=(0, 2, 3)), rtol=2e-2)
+
+
+@pytest.mark.parametrize("s,p,d", [(1, 1, 1), (2, 0, 1), (1, 2, 2), (3, 1, 2)])
+def test_conv1d_layouts_against_torch(s, p, d):
+    X, F = _rand((2, 19, 6), 5), _rand((3, 6, 4), 6)                                  # NWC, (K,CI,CO)
+    ref = torch.nn.functional.conv1d(torch.from_numpy(X.astype(np.float64)).permute(0, 2, 1),
+                                     torch.from_numpy(F.astype(np.float64)).permute(2, 1, 0), stride=s, padding=p, dilation=d)
+    got = oracle.conv1d_nwc_ref(X, F, s, p, d)
+    assert np.allclose(got, ref.permute(0, 2, 1).numpy())
+    got2 = oracle.conv1d_ncw_ref(X.transpose(0, 2, 1), F.transpose(2, 1, 0), s, p, d)
+    assert np.allclose(got2, ref.numpy())
+
+
+@pytest.mark.parametrize("s,p,d", [(1, 1, 1), ((2, 1), (0, 2), 1), (1, 2, 2)])
+def test_conv2d_nchw_and_dil_against_torch(s, p, d):
+    X, F = _rand((2, 3, 9, 8), 7), _rand((5, 3, 3, 3), 8)
+    ref = torch.nn.functional.conv2d(torch.from_numpy(X.astype(np.float64)), torch.from_numpy(F.astype(np.float64)),
+                                     stride=s, padding=p, dilation=d).numpy()
+    assert np.allclose(oracle.conv2d_nchw_ref(X, F, s, p, d), ref)
+    got = oracle.dil_nhwc_ref(X.transpose(0, 2, 3, 1), F.transpose(2, 3, 1, 0), s, p, d)
+    assert np.allclose(got, ref.transpose(0, 2, 3, 1))
+
+
+@pytest.mark.parametrize("s,p,d", [(1, 1, 1), ((2, 1, 1), (1, 0, 1), 1), (1, (0, 2, 1), (1, 2, 1))])
+def test_conv3d_layouts_against_torch(s, p, d):
+    X, F = _rand((2, 4, 6, 7, 5), 9), _rand((6, 4, 3, 3, 2), 10)                     # NCDHW, (CO,CI,KD,KH,KW)
+    ref = torch.nn.functional.conv3d(torch.from_numpy(X.astype(np.float64)), torch.from_numpy(F.astype(np.float64)),
+                                     stride=s, padding=p, dilation=d).numpy()
+    assert np.allclose(oracle.conv3d_ncdhw_ref(X, F, s, p, d), ref)
+    got = oracle.conv3d_ndhwc_ref(X.transpose(0, 2, 3, 4, 1), F.transpose(2, 3, 4, 1, 0), s, p, d)
+    assert np.allclose(got, ref.transpose(0, 2, 3, 4, 1))
+
+
+@pytest.mark.parametrize("s,p,d,op", [(1, 0, 1, 0), (2, 1, 1, 1), (2, 1, 1, 0), (3, 2, 2, 1), (1, 1, 2, 0)])
+def test_conv2d_transposed_against_torch(s, p, d, op):
+    """The declaration (expand, pad, unflipped stride-1 correlation) is a transposed convolution whose torch weight
+    is the filter flipped in both window axes with the channel axes swapped."""
+    X, F = _rand((2, 4, 5, 6), 11), _rand((3, 4, 3, 4), 12)                           # (N,CI,H,W), (CO,CI,KH,KW)
+    w = torch.from_numpy(F.astype(np.float64)).flip(2, 3).permute(1, 0, 2, 3)        # (CI,CO,KH,KW)
+    ref = torch.nn.functional.conv_transpose2d(torch.from_numpy(X.astype(np.float64)), w, stride=s, padding=p,
+                                               output_padding=op, dilation=d).numpy()
+    got = oracle.conv2d_transposed_nchw_ref(X, F, s, p, d, op)
+    assert got.shape == ref.shape and np.allclose(got, ref)

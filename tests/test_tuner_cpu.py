@@ -213,3 +213,34 @@ def test_cost_model_learns_and_ranks():
     assert np.corrcoef(pred, y)[0, 1] > 0.95
     score = m.bst.get_score()
     assert max(score, key=score.get) in ("f0", "f3")
+
+
+@pytest.mark.parametrize("op,shape", [("gemv", [4096, 4096]), ("scan", [512, 512, 512]), ("mean", [32, 64, 56, 56]),
+                                      ("var", [32, 64, 56, 56]), ("c1d", [32, 1024, 64, 128, 3, 1, 1, 1]),
+                                      ("c1d_nwc", [32, 1024, 64, 128, 3, 2, 1, 2]),
+                                      ("c2d_nchw", [32, 224, 224, 3, 64, 7, 7, 2, 3, 1]),
+                                      ("dil", [16, 56, 56, 64, 64, 3, 3, 1, 2, 2]),
+                                      ("c3d", [16, 8, 28, 28, 16, 32, 3, 3, 3, 1, 1, 1]),
+                                      ("c3d_ndhwc", [16, 8, 28, 28, 16, 32, 3, 3, 3, (2, 1, 1), 1, 1]),
+                                      ("t2d", [16, 14, 14, 64, 32, 4, 4, 2, 1, 1, 0])])
+def test_registry_operators_have_a_feasible_template_space(op, shape):
+    """Every operator of the registry (ops/cuda/__init__.py:15-32 names) yields a tunable space on the MFMA templates
+    whose samples the C side accepts, and announces kernel operands of the GEMM / conv view it declares."""
+    cfg = Config()
+    cfg.codegen_type = 'GPU_MFMA'
+    t = Task("t", getOpFromName(op), shape + ["float16", "float16"], "rocm")
+    t.config = cfg
+    t.make_stage_schedules()
+    seen = set()
+    for _ in range(6):
+        km = copy.deepcopy(t.knob_manager)
+        valid, _ = km.randSample({})
+        s, args = t.instantiate(km)
+        d = s.to_desc()
+        assert valid and B.check_desc(d), (d, B.lib().hrn_last_error())
+        seen.add(d.as_tuple())
+        g = s.info['gemm_view']
+        p = s.to_problem()
+        assert (p.m, p.n, p.k) == (g['M'], g['N'], g['K'])
+        assert s.info['adapter'] in __import__('heron_amd.hostops', fromlist=['ADAPTERS']).ADAPTERS
+    assert len(seen) >= 3
