@@ -8,7 +8,8 @@ from .runner.measure import create_measure_batch
 from .runner.runner import Runner
 from .schedule.sched_op import get_op_methods
 from .task.task import Task
-from .tuner import CGATuner, CRandSampler, CRandTuner, GATuner, RCGATuner
+from .tuner import (CGATuner, ConstrainedRandomWalkerSATuner, CRandSampler, CRandTuner, GATuner, IDEATuner, RCGATuner,
+                    RandomWalkSATuner, SDGATuner, SRGATuner)
 from .utils import mkdir
 
 
@@ -59,7 +60,9 @@ class Env:
 
         self.config.setEnv(self)
         method = self.config.opt_method
-        tuners = {'CRAND': CRandTuner, 'CRANDS': CRandSampler, 'CGA': CGATuner, 'RCGA': RCGATuner, 'GA': GATuner}
+        tuners = {'CRAND': CRandTuner, 'CRANDS': CRandSampler, 'CGA': CGATuner, 'RCGA': RCGATuner, 'GA': GATuner,
+                  'SRGA': SRGATuner, 'SDGA': SDGATuner, 'IDEA': IDEATuner, 'SA': RandomWalkSATuner,
+                  'CSA': ConstrainedRandomWalkerSATuner}
         if method not in tuners:
             raise ValueError('Unsupportted opt method')
         self.tuner = tuners[method](self.config)

@@ -298,6 +298,35 @@ class KnobManager:
             self.solved_knob_vals_phenotype[key] = phenotype[idx]
         return phenotype, valid
 
+    def SBX_crossover_and_mutation(self, m1, m2, feasible, eta_c=15, eta_m=20, p_mut=0.1):
+        """Simulated-binary crossover and polynomial mutation over ALL variables, each result snapped to the nearest
+        value seen feasible for that variable; the child may violate constraints and carries the per-constraint
+        violations for the infeasibility-driven ranking (knobManager.py:392-430)."""
+        chrom, res = {}, []
+        for key in m1.solved_knob_vals_genotype.keys():
+            x1, x2 = m1.solved_knob_vals_genotype[key], m2.solved_knob_vals_genotype[key]
+            cands = feasible[key]
+            u = random.random()
+            if u <= 0.5:
+                beta = (2 * u) ** (1.0 / eta_c + 1)
+            else:
+                beta = (1.0 / (2 * (1 - u + 1e-8))) ** (1.0 / eta_c + 1)
+            beta *= random.choice((-1.0, 1.0))
+            x = 0.5 * ((1 + beta) * x1 + (1 - beta) * x2)
+            x = min(cands, key=lambda t: abs(t - x))
+            if random.random() < p_mut:
+                span = max(cands) - min(cands)
+                r = random.random()
+                delta = (2 * r) ** (1.0 / (eta_m + 1)) - 1 if r < 0.5 else 1 - (2 * (1 - r)) ** (1.0 / (eta_m + 1))
+                x = min(cands, key=lambda t: abs(t - (x + span * delta)))
+            chrom[key] = x
+            res.append(x)
+        violations, valid = self.solver.MultiSATScore(chrom)
+        self.solved_knob_vals_genotype = chrom
+        self.solved_knob_vals_phenotype = chrom
+        self._valid = valid
+        return res, valid, violations
+
     def constrained_random_walk(self, knob_manager, ratio):
         """Keep a random ``ratio`` of the parent's values, re-solve the rest (knobManager.py:433-444)."""
         keys = list(knob_manager.solved_knob_vals_genotype.keys())

@@ -148,8 +148,10 @@ class tileWaveOp(schedOp):
 
 
 class tileBlockOp(schedOp):
-    """Workgroup tile: M = grid_m * bm, bm = wm * wave_tile_m (and the same for N), the ProdTwo chain of
-    a two-level split (knobManager.py:83-107)."""
+    """Workgroup tile: bm = wm * wave_tile_m and grid_m = ceil(M / bm) (and the same for N).  The reference's split
+    chain is exact (extent = outer * inner, knobManager.py:83-107) because TVM splits must divide; the kernel
+    guards ragged edge tiles itself, so the chain here is the covering form
+    grid * b = extent + waste, 0 <= waste < b, which keeps shapes with awkward factors (149 * 149 pixels) tunable."""
 
     def perform(self, s, stage_name, ctx):
         km = ctx.knob_manager
@@ -159,14 +161,19 @@ class tileBlockOp(schedOp):
             bkey = self.var(ctx, stage_name, b, 16, min(512, extent), 16)
             gkey = self.var(ctx, stage_name, g, 1, extent // 16, extent // 16)
             km.addProd([self.P(stage_name, w), self.V(stage_name, wt)], bkey)
-            km.addProd([gkey, bkey], extent)
+            cover = self.var(ctx, stage_name, g + '_cover', extent, extent + 511, extent)
+            waste = self.var(ctx, stage_name, g + '_waste', 0, 511, 0)
+            km.addProd([gkey, bkey], cover)
+            km.addSUM(cover, [extent, waste])
+            km.addLT(waste, bkey)
             s.params['bm' if ax == 'i' else 'bn'] = km.get_val(bkey)
         ctx.addSchedDesc("block tile = %s x %s\n" % (s.params['bm'], s.params['bn']))
 
 
 class tileKOp(schedOp):
-    """K tiling: bkb bytes of K per LDS row, an even number >= 2 of MFMA k-steps per tile, and K an exact
-    multiple of the tile (the split constraint of the reduce axis, sched_common.py generalTileOp)."""
+    """K tiling: bkb bytes of K per LDS row, an even number >= 2 of MFMA k-steps per tile, and k_tiles =
+    ceil(K_bytes / bkb) (the split constraint of the reduce axis, sched_common.py generalTileOp, in covering form:
+    the part of the last tile past the end of K is fetched as zeros)."""
 
     def perform(self, s, stage_name, ctx):
         km = ctx.knob_manager
@@ -176,7 +183,11 @@ class tileKOp(schedOp):
         km.addCandidates(ks, [2, 4, 8])
         km.addProd([ks, self.V(stage_name, 'mfma_k_bytes')], bkb)
         kt = self.var(ctx, stage_name, 'k_tiles', 1, kbytes // 64, kbytes // 64)
-        km.addProd([kt, bkb], kbytes)
+        kcover = self.var(ctx, stage_name, 'k_cover', kbytes, kbytes + 255, kbytes)
+        kwaste = self.var(ctx, stage_name, 'k_waste', 0, 255, 0)
+        km.addProd([kt, bkb], kcover)
+        km.addSUM(kcover, [kbytes, kwaste])
+        km.addLT(kwaste, bkb)
         s.params['bkb'] = km.get_val(bkb)
         ctx.addSchedDesc("k tile = %s bytes\n" % s.params['bkb'])
 

@@ -111,6 +111,59 @@ class RCGATuner(GATuner):
         return res
 
 
+class SRGATuner(GATuner):
+    """GA over all variables without constraint handling in the operators; constraint pressure comes from
+    stochastic ranking: a bubble sort whose comparisons use the predicted score when both neighbours are feasible
+    or with probability ``pf``, and the total violation otherwise (ga_tuner.py:113-154)."""
+    SWEEPS, PF = 10, 0.45
+
+    def Selection(self, pop, num):
+        return self.RankSelection(pop, num)
+
+    def RankPop(self, pop):
+        order = list(pop)
+        for _ in range(self.SWEEPS):
+            swapped = False
+            for j in range(len(order) - 1):
+                a, b = order[j], order[j + 1]
+                va, vb = a.violation or 0, b.violation or 0
+                if (va == 0 and vb == 0) or random.random() < self.PF:
+                    out_of_order = a.predict < b.predict
+                else:
+                    out_of_order = va > vb
+                if out_of_order:
+                    order[j], order[j + 1] = b, a
+                    swapped = True
+            if not swapped:
+                break
+        return order
+
+    def crossoverAndMutate(self, samples, task):
+        res = _offspring(self.config, 'UnconstrainedAll', samples, task, self.feasible)
+        perfs = self.predict(res)
+        for idx, sample in enumerate(res):
+            sample.predict = perfs[idx]
+        return res
+
+
+class SDGATuner(GATuner):
+    """GA whose genotype is decoded into a feasible phenotype by repairing it with the solver
+    (SAT-decoding, ga_tuner.py:157-166)."""
+
+    def crossoverAndMutate(self, samples, task):
+        res = _offspring(self.config, 'SATDecoding', samples, task, self.feasible)
+        perfs = self.predict(res)
+        for idx, sample in enumerate(res):
+            sample.predict = perfs[idx]
+        return res
+
+
+def _offspring(config, kind, samples, task, extra):
+    if config.parallel:
+        return crossoverAndMutateParallel(kind, config.pop_num, samples, task, config.parallel_num, extra)
+    return crossoverAndMutateSequential(kind, config.pop_num, samples, task, extra)
+
+
 def crossoverAndMutateParallel(kind, number, population, task, parallel_num, extra, timeout=60):
     work_load = int((number + parallel_num - 1) // parallel_num)
     jobs = [Job(crossoverAndMutateSequential, (kind, work_load, population, task, extra), timeout)
@@ -130,6 +183,12 @@ def crossoverAndMutateSequential(kind, number, population, task, extra):
         child = Sample(task)
         if kind == 'Constrained':
             point, valid = child.knob_manager.constrained_crossover_and_mutate(m1.knob_manager, m2.knob_manager, extra)
+        elif kind == 'UnconstrainedAll':
+            point, valid, child.violation = child.knob_manager.crossover_and_mutate_all(m1.knob_manager, m2.knob_manager, extra)
+        elif kind == 'SATDecoding':
+            point, valid = child.knob_manager.satdecoding_crossover_and_mutate(m1.knob_manager, m2.knob_manager, extra)
+        elif kind == 'SBX':
+            point, valid, child.violations = child.knob_manager.SBX_crossover_and_mutation(m1.knob_manager, m2.knob_manager, extra)
         else:
             point, valid = child.knob_manager.crossover_and_mutate(m1.knob_manager, m2.knob_manager, extra)
         child.point = point

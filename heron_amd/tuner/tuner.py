@@ -59,7 +59,9 @@ class Tuner:
             sample_e = time.time()
 
             measure_s = time.time()
-            pop = self.epsilon_select(env, all_pop, 0.6, select_num)
+            # points known to violate the constraint system are not worth a build (the reference selects among them
+            # too and lets the build fail, tuner.py:66-70)
+            pop = self.epsilon_select(env, [x for x in all_pop if x.valid], 0.6, select_num)
             if do_measure and pop != []:
                 samples = self.FilterSamples(pop, env)
                 self.measure(samples, env)

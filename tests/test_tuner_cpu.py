@@ -8,6 +8,7 @@ import copy
 import json
 import math
 import os
+import random
 import time
 
 import numpy as np
@@ -102,7 +103,7 @@ def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
         d = s.to_desc()
         assert valid and B.check_desc(d), (d, B.lib().hrn_last_error())
         g = s.info['gemm_view']
-        assert g['M'] <= math.ceil(g['M'] / d.bm) * d.bm and (16 * math.ceil(g['M'] / 16)) % d.bm == 0
+        assert d.bm <= 16 * math.ceil(g['M'] / 16) and d.bn <= 16 * math.ceil(g['N'] / 16)
         vals = km.solved_knob_vals_phenotype
         lds_key = [k for k in km.solver.vals if k.endswith("VA:lds_bytes_total")] or \
                   [k for k in km.solver.vals if k.endswith("VA:lds_bytes")]
@@ -244,3 +245,68 @@ def test_registry_operators_have_a_feasible_template_space(op, shape):
         assert (p.m, p.n, p.k) == (g['M'], g['N'], g['K'])
         assert s.info['adapter'] in __import__('heron_amd.hostops', fromlist=['ADAPTERS']).ADAPTERS
     assert len(seen) >= 3
+
+
+@pytest.mark.parametrize("method", ["GA", "SRGA", "SDGA", "IDEA", "SA", "CSA", "RCGA"])
+def test_baseline_tuners_run_and_only_measure_feasible_points(tmp_path, method):
+    """The comparison tuners of the reference's ablations (environment.py:68-91): each completes a run on the CDNA4
+    space, every measured record is a feasible point of the CSP, and the search beats the worst tile of the model."""
+    env = make_env(tmp_path, method=method, trials=40)
+    random.seed(1)
+    np.random.seed(1)
+    env.tune("T1")
+    rows = [json.loads(l) for l in open(os.path.join(env.config.log_dir, "records.txt"))]
+    assert 8 <= len(rows) <= 56           # three full rounds of 16 plus the 40 % 16 remainder round (tuner.py:50-58)
+    solver = env.task.knob_manager.solver
+    for r in rows:
+        assert solver.SATScore(r["param"]) == 0
+    assert math.exp(-max(r["perf"] for r in rows)) < 3.0e-3
+    if method in ("GA", "SRGA", "SDGA", "IDEA", "SA"):
+        assert os.path.exists(env.config.feasible_file_path)     # per-variable feasible values were sampled first
+
+
+class _S:
+    def __init__(self, predict, violation=0, valid=True, violations=None):
+        self.predict, self.violation, self.valid, self.violations = predict, violation, valid, violations
+
+
+def test_stochastic_ranking_prefers_feasible_then_score():
+    from heron_amd.tuner import SRGATuner
+    t = SRGATuner.__new__(SRGATuner)
+    random.seed(0)
+    # all feasible: plain sort by predicted score, best first
+    pop = [_S(p) for p in (1.0, 5.0, 3.0, 4.0, 2.0)]
+    assert [s.predict for s in t.RankPop(pop)] == [5.0, 4.0, 3.0, 2.0, 1.0]
+    # pf = 0: infeasible neighbours are ordered by violation only, so the heavy violator sinks below the light one
+    t.PF = 0.0
+    pop = [_S(9.0, violation=50), _S(1.0, violation=2), _S(2.0, violation=0)]
+    ranked = t.RankPop(pop)
+    assert [s.violation for s in ranked] == [0, 2, 50]
+
+
+def test_idea_rank_fronts_and_sa_acceptance():
+    from heron_amd.tuner import IDEATuner, RandomWalkSATuner
+
+    class KM:
+        class solver:
+            primitives = [0, 1]
+    t = IDEATuner.__new__(IDEATuner)
+    # (predict, violations): a dominates c (better score, smaller violations); b trades score for violation
+    a, b, c = _S(5.0, valid=False, violations=[1, 1]), _S(6.0, valid=False, violations=[3, 3]), _S(4.0, valid=False, violations=[2, 2])
+    for s in (a, b, c):
+        s.knob_manager = KM
+    ranked = t.Rank([c, b, a])
+    # objectives are (predict, rank-sum) with larger dominating (idea_tuner.py:96-98): b has the top score and the
+    # top rank-sum so it alone forms the first front
+    assert ranked[0] is b and {id(x) for x in ranked} == {id(a), id(b), id(c)}
+    sa = RandomWalkSATuner.__new__(RandomWalkSATuner)
+    np.random.seed(0)
+    cur = [_S(1.0) for _ in range(200)]
+    better = [_S(2.0) for _ in range(200)]
+    worse = [_S(0.5) for _ in range(200)]
+    bad = [_S(9.0, valid=False) for _ in range(200)]
+    assert all(x.predict == 2.0 for x in sa.accept(cur, better, 0.5))             # improvements always accepted
+    frac = np.mean([x.predict == 0.5 for x in sa.accept(cur, worse, 0.5)])
+    assert 0.2 < frac < 0.55                                                         # exp(-0.5/0.5) = 0.37
+    assert np.mean([x.predict == 0.5 for x in sa.accept(cur, worse, 0.0)]) == 0      # frozen: never
+    assert all(x.predict == 1.0 for x in sa.accept(cur, bad, 0.5))                   # infeasible steps rejected
