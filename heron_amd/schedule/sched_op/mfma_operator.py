@@ -134,11 +134,11 @@ class tileWaveOp(schedOp):
         wn = self.knob(ctx, stage_name, 'wave_n', [1, 2, 4, 8], 2)
         waves = self.var(ctx, stage_name, 'waves', 1, max_waves, 4)
         km.addProd([wm, wn], waves)
-        tm = self.knob(ctx, stage_name, 'tile_m', list(range(1, 9)), 2)
-        tn = self.knob(ctx, stage_name, 'tile_n', list(range(1, 9)), 2)
+        tm = self.knob(ctx, stage_name, 'tile_m', list(range(1, 17)), 2)
+        tn = self.knob(ctx, stage_name, 'tile_n', list(range(1, 17)), 2)
         mfma = self.P(stage_name, 'mfma')
-        wtm = self.var(ctx, stage_name, 'wave_tile_m', 16, 256, 64)
-        wtn = self.var(ctx, stage_name, 'wave_tile_n', 16, 256, 64)
+        wtm = self.var(ctx, stage_name, 'wave_tile_m', 16, 512, 64)
+        wtn = self.var(ctx, stage_name, 'wave_tile_n', 16, 512, 64)
         km.addProd([tm, mfma], wtm)
         km.addProd([tn, mfma], wtn)
         for k, key in (('wm', wm), ('wn', wn), ('tm', tm), ('tn', tn)):
@@ -344,13 +344,13 @@ class registerBudgetOp(schedOp):
         regs_total = ctx.getLimit('regs_per_simd_lane')
         simds = ctx.getLimit('simd_per_cu')
         tm, tn = self.P(stage_name, 'tile_m'), self.P(stage_name, 'tile_n')
-        tmn = self.var(ctx, stage_name, 'tiles_per_wave', 1, 64, 4)
+        tmn = self.var(ctx, stage_name, 'tiles_per_wave', 1, 128, 4)
         km.addProd([tm, tn], tmn)
         acc = self.var(ctx, stage_name, 'acc_regs', 4, regs_total // 2, 64)
         km.addProd([tmn, self.V(stage_name, 'acc_regs_per_tile')], acc)
-        tsum = self.var(ctx, stage_name, 'tile_m_plus_n', 2, 16, 4)
+        tsum = self.var(ctx, stage_name, 'tile_m_plus_n', 2, 32, 4)
         km.addSUM(tsum, [tm, tn])
-        frag = self.var(ctx, stage_name, 'frag_regs', 16, 128, 32)
+        frag = self.var(ctx, stage_name, 'frag_regs', 16, 256, 32)
         km.addProd([8, tsum], frag)
         regs = self.var(ctx, stage_name, 'regs_per_lane', 1, regs_total, 128)
         km.addSUM(regs, [acc, frag, self.OVERHEAD])
