@@ -61,6 +61,15 @@ def make_workloads(torch, workloads, instances):
     ops, byts = workloads.conv_work(32, 56, 56, 64, 64, 3, 3, 1, 1, 1)
     W["conv2d_f16_resnet"] = dict(desc=instances.BEST["conv2d_f16"], build=build_conv, ops=ops, bytes=byts, f16=True,
                                   desc_text="conv2d_nhwc_f16 N=32 H=W=56 C=64 K=64 3x3 s1 p1")
+
+    def build_conv_i8():
+        X, Wt = workloads.conv2d_u8s8_inputs(32, 56, 56, 64, 64, 3, 3, seed=6)
+        Y = torch.empty((32, 56, 56, 64), dtype=torch.int32, device="cuda")
+        return dev(X), dev(Wt), Y, B.conv2d_problem(32, 56, 56, 64, 64, 3, 3, 1, 1, 1,
+                                                    instances.BEST_GROUP_M.get("conv2d_u8s8", 8))
+    ops, byts = workloads.conv_work(32, 56, 56, 64, 64, 3, 3, 1, 1, 1, in_bytes=1, out_bytes=4)
+    W["conv2d_u8s8_resnet"] = dict(desc=instances.BEST["conv2d_u8s8"], build=build_conv_i8, ops=ops, bytes=byts, f16=False,
+                                   desc_text="conv2d_nhwc_u8s8 N=32 H=W=56 C=64 K=64 3x3 s1 p1")
     return W
 
 
@@ -174,8 +183,8 @@ def cpu_baseline(name, workloads):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="gemm_f16_4096")
     ap.add_argument("--only", action="store_true", help="skip the 'also' workloads and the CPU baseline")
     ap.add_argument("--probe", action="store_true", help="only run the roofline probes (MFMA loop, 1 GiB copy)")
@@ -223,7 +232,7 @@ def main():
         for name, ww in W.items():
             if name == args.workload:
                 continue
-            steps = max(10, min(args.steps, 50))
+            steps = max(10, min(args.steps, 500))
             wl, e, _ = measure(torch, B, ww, steps, min(args.warmup, 5))
             r = roofline(ww, e, workloads)
             also.append({"workload": ww["desc_text"], "value": ww["ops"] / wl / 1e12,

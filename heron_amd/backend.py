@@ -50,10 +50,10 @@ class KernelDesc(ctypes.Structure):
                 ("bkb", ctypes.c_int32), ("wm", ctypes.c_int32), ("wn", ctypes.c_int32), ("mfma", ctypes.c_int32),
                 ("stages", ctypes.c_int32), ("swizzle", ctypes.c_int32), ("epilogue", ctypes.c_int32),
                 ("waves_per_eu", ctypes.c_int32), ("l2_prefetch", ctypes.c_int32), ("ablate", ctypes.c_int32),
-                ("load_mode", ctypes.c_int32), ("conv_window", ctypes.c_int32)]
+                ("load_mode", ctypes.c_int32), ("conv_window", ctypes.c_int32), ("persistent", ctypes.c_int32)]
 
     KEYS = ("dtype", "op", "bm", "bn", "bkb", "wm", "wn", "mfma", "stages", "swizzle", "epilogue", "waves_per_eu",
-            "l2_prefetch", "ablate", "load_mode", "conv_window")
+            "l2_prefetch", "ablate", "load_mode", "conv_window", "persistent")
 
     def as_tuple(self):
         return tuple(int(getattr(self, k)) for k in self.KEYS)
@@ -84,9 +84,10 @@ class Problem(ctypes.Structure):
 
 
 def make_desc(dtype, op=HRN_OP_GEMM, bm=128, bn=128, bkb=128, wm=2, wn=2, mfma=32, stages=2, swizzle=1,
-              epilogue=0, waves_per_eu=0, l2_prefetch=0, ablate=0, load_mode=0, conv_window=0):
+              epilogue=0, waves_per_eu=0, l2_prefetch=0, ablate=0, load_mode=0, conv_window=0, persistent=0):
     d = KernelDesc()
     d.l2_prefetch, d.ablate, d.load_mode, d.conv_window = l2_prefetch, ablate, load_mode, conv_window
+    d.persistent = persistent
     d.dtype, d.op, d.bm, d.bn, d.bkb, d.wm, d.wn = dtype, op, bm, bn, bkb, wm, wn
     d.mfma, d.stages, d.swizzle, d.epilogue, d.waves_per_eu = mfma, stages, swizzle, epilogue, waves_per_eu
     return d

@@ -36,6 +36,7 @@ class Config:
         self.temperature = 0.6
 
         self.feasible_file_path = 'feasible.json'
+        self.feasible_samples = 1000          # random feasible points behind the per-variable value sets (tuner.py:115)
 
         # defaults for configs created in code rather than from a file
         self.opt_method = 'CGA'

@@ -46,6 +46,7 @@ struct hrn_module {
     hipModule_t mod;
     hipFunction_t fn;
     std::string path;
+    int persist_grid;   // persistent instances: workgroups that fit the device at once (multiple of 8 when >= 8)
 };
 
 namespace {
@@ -125,6 +126,9 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (d->conv_window && (d->op != HRN_OP_CONV2D || d->load_mode || d->l2_prefetch))
         return fail(HRN_E_BADPARAM, "conv_window is a conv2d option (load_mode 0, no l2_prefetch)");
     if (d->load_mode == 1 && (d->stages != 2 || d->l2_prefetch)) return fail(HRN_E_BADPARAM, "load_mode 1 needs stages == 2 and no l2_prefetch");
+    if (d->persistent < 0 || d->persistent > 1) return fail(HRN_E_BADPARAM, "persistent %d", d->persistent);
+    if (d->persistent && (d->epilogue != 1 || d->load_mode || d->l2_prefetch || d->conv_window || d->ablate))
+        return fail(HRN_E_BADPARAM, "persistent needs the LDS-staged epilogue and none of load_mode, l2_prefetch, conv_window, ablate");
     Derived r;
     r.es = d->dtype == HRN_DT_F16 ? 2 : 1;
     r.nw = d->wm * d->wn;
@@ -151,7 +155,15 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
         const int base = d->dtype == HRN_DT_U8S8 ? ((d->bn * 4 + 1023) / 1024) * 1024 : 0;
         const int epi = base + r.nw * d->mfma * (wtn * oes + 16);
         if ((d->mfma * (wtn * oes / 16)) % 64) return fail(HRN_E_BADPARAM, "staged epilogue needs mfma*wave_tile_n*out_bytes/16 %% 64 == 0");
-        r.lds = std::max(r.lds, epi);
+        if (d->persistent) {
+            // the stages stay live during the epilogue, and its stores share the 6-bit vector-memory counter with the fetches
+            r.lds += epi;
+            const int stores = r.tm * (d->mfma * (wtn * oes / 16) / 64);
+            if ((d->stages - 2) * r.lpt + stores > 63)
+                return fail(HRN_E_BADPARAM, "persistent: %d fetches + %d stores in flight exceed 63", (d->stages - 2) * r.lpt, stores);
+        } else {
+            r.lds = std::max(r.lds, epi);
+        }
     }
     if (r.lds > 163840) return fail(HRN_E_BADPARAM, "LDS %d > 163840", r.lds);
     if (d->swizzle && (r.cpr << (d->swizzle - 1)) > d->mfma)
@@ -175,8 +187,9 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
 
 std::string desc_key(const hrn_kernel_desc* d, uint64_t srch) {
     char b[256];
-    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_a%d_f%d_l%d_c%d_%08x", d->dtype, d->op, d->bm, d->bn,
+    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_a%d_f%d_l%d_c%d_r%d_%08x", d->dtype, d->op, d->bm, d->bn,
              d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu, d->ablate, d->l2_prefetch, d->load_mode, d->conv_window,
+             d->persistent,
              (unsigned)(srch ^ (srch >> 32)));
     return b;
 }
@@ -256,6 +269,7 @@ int compile_desc(const hrn_kernel_desc* d, double timeout_s, std::string* out_pa
     def("HRN_PF", d->l2_prefetch);
     def("HRN_LOAD", d->load_mode);
     def("HRN_CONVWIN", d->conv_window);
+    def("HRN_PERSIST", d->persistent);
     args.push_back(src);
     args.push_back("-o");
     args.push_back(co_tmp);
@@ -358,6 +372,18 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
     const int64_t total = (int64_t)k->tiles_m * k->tiles_n * p->batch;
     if (total <= 0 || total >= (1ll << 31)) return fail(HRN_E_BADPARAM, "grid size");
     *grid = (unsigned)total;
+    if (d.persistent) {
+        const int oes = d.dtype == HRN_DT_F16 ? 2 : 4;
+        if ((int64_t)p->n * oes % 16) return fail(HRN_E_BADPARAM, "persistent instances store whole 16-byte chunks: N*%d must be a multiple of 16", oes);
+        if ((int64_t)p->m * p->ldc * oes >= (1ll << 31)) return fail(HRN_E_BADPARAM, "persistent: C exceeds 2 GiB per batch entry");
+        int64_t g = std::min<int64_t>(total, mod->persist_grid);
+        if (const char* e = getenv("HRN_PERSIST_GRID")) {      // override of the number of workgroups (tuning / tests)
+            const long v = atol(e);
+            if (v >= 1) g = std::min<int64_t>(total, v);
+        }
+        if (g >= 8) g &= ~7ll;          // workgroup i runs on XCD i % 8: keep tile t on XCD t % 8 in every round
+        *grid = (unsigned)g;
+    }
     return HRN_OK;
 }
 
@@ -449,7 +475,12 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(float* sink, int iters,
 
 __global__ void __launch_bounds__(256) probe_copy_kernel(const pv4i* __restrict__ src, pv4i* __restrict__ dst, size_t n16) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i + 3 * stride < n16; i += 4 * stride) {      // four independent 16-byte loads in flight per lane
+        const pv4i v0 = src[i], v1 = src[i + stride], v2 = src[i + 2 * stride], v3 = src[i + 3 * stride];
+        dst[i] = v0; dst[i + stride] = v1; dst[i + 2 * stride] = v2; dst[i + 3 * stride] = v3;
+    }
+    for (; i < n16; i += stride) dst[i] = src[i];
 }
 
 }  // namespace
@@ -583,6 +614,18 @@ int hrn_build(const hrn_kernel_desc* desc, double timeout_s, hrn_module** out) {
         (void)hipModuleUnload(m->mod);
         delete m;
         return fail(HRN_E_LOAD, "hipModuleGetFunction: %s", hipGetErrorString(e));
+    }
+    m->persist_grid = 0;
+    if (desc->persistent) {
+        int per_cu = 0, dev = 0;
+        hipDeviceProp_t pr;
+        if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, m->fn, m->info.threads, 0) != hipSuccess || per_cu < 1 ||
+            hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&pr, dev) != hipSuccess) {
+            (void)hipModuleUnload(m->mod);
+            delete m;
+            return fail(HRN_E_LOAD, "occupancy query failed: %s", hipGetErrorString(hipGetLastError()));
+        }
+        m->persist_grid = per_cu * pr.multiProcessorCount;
     }
     *out = m;
     return HRN_OK;

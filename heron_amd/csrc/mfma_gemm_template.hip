@@ -85,6 +85,16 @@ constexpr int LOADM = HRN_LOAD;
 #define HRN_CONVWIN 0
 #endif
 constexpr bool CW = (HRN_CONVWIN != 0);
+// Persistent mode: the launch has fewer workgroups than output tiles and every workgroup walks tiles
+// blockIdx.x, blockIdx.x + gridDim.x, ...  The k-tiles of all its output tiles form ONE stream through the LDS
+// stages, so the first k-tiles of the next output tile are already being fetched while the current tile's result is
+// stored.  The stores are buffer stores issued unconditionally (masked lanes get an out-of-range offset), so every
+// wave has a known number of them in the vector-memory counter and the waits on the following tile fetches can
+// allow for them instead of draining them.
+#ifndef HRN_PERSIST
+#define HRN_PERSIST 0
+#endif
+constexpr bool PERS = (HRN_PERSIST != 0);
 constexpr int ES = (DT == 0) ? 2 : 1;       // input element bytes
 constexpr int OES = (DT == 0) ? 2 : 4;      // output element bytes
 constexpr int NW = WM * WN, NT = NW * 64;
@@ -119,7 +129,13 @@ constexpr int PF_SCRATCH = PF ? NW * 256 : 0;                   // LDS corner th
 constexpr int EPI_PITCH = WTN * OES + 16;
 constexpr int EPI_BASE = (DT == 1) ? ((BN * 4 + 1023) / 1024) * 1024 : 0;
 constexpr int EPI_BYTES = (EPI == 1) ? EPI_BASE + NW * MT * EPI_PITCH : 0;
-constexpr int LDS_BYTES = (NS * STAGE_BYTES + PF_SCRATCH > EPI_BYTES) ? NS * STAGE_BYTES + PF_SCRATCH : EPI_BYTES;
+// the epilogue region (column sums + strips) reuses the stages, except in persistent mode where the stages stay live
+constexpr int EPI_OFF = PERS ? NS * STAGE_BYTES : 0;
+constexpr int LDS_BYTES = PERS ? NS * STAGE_BYTES + EPI_BYTES
+                               : ((NS * STAGE_BYTES + PF_SCRATCH > EPI_BYTES) ? NS * STAGE_BYTES + PF_SCRATCH : EPI_BYTES);
+constexpr int STORES_PER_TILE = (EPI == 1) ? TM * (MT * (WTN * OES / 16) / 64) : 0;   // store instructions per wave per output tile
+static_assert(!PERS || (EPI == 1 && LOADM == 0 && PF == 0 && !CW && HRN_ABLATE == 0), "persistent mode: staged epilogue, direct loads");
+static_assert(!PERS || (NS - 2) * (A_LPW + B_LPW) + STORES_PER_TILE <= 63, "persistent mode: vmcnt range");
 static_assert(LDS_BYTES <= 163840, "LDS");
 static_assert(EPI == 0 || (MT * (WTN * OES / 16)) % 64 == 0, "staged epilogue: a strip must split into whole wave stores");
 static_assert(SWZ == 0 || (CPR << (SWZ - 1)) <= MT, "swizzle period must fit in one MFMA tile");
@@ -212,79 +228,95 @@ hrn_mfma_kernel(const HrnKArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm_idx = wave / WN, wn_idx = wave % WN;
 
-    // ---- tile raster: spread over the 8 XCDs so that each XCD's L2 sees a compact block ----
     const int tiles_mn = a.tiles_m * a.tiles_n;
     const int total = tiles_mn * a.batch;
-    int pid = blockIdx.x;
-    if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
-    const int bz = pid / tiles_mn;
-    const int t = pid - bz * tiles_mn;
-    const int group_sz = a.group_m * a.tiles_n;
-    const int gid = t / group_sz;
-    const int first_m = gid * a.group_m;
-    const int gsz = min(a.tiles_m - first_m, a.group_m);
-    const int tin = t - gid * group_sz;
-    const int tile_m = first_m + tin % gsz;
-    const int tile_n = tin / gsz;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-
-    const char* Ab = (const char*)a.A + (int64_t)bz * a.sA * ES;
-    const char* Bb = (const char*)a.B + (int64_t)bz * a.sB * ES;
     const uint32_t Kb = (uint32_t)a.K * ES;           // bytes of K
     const int KT = (Kb + BKB - 1) / BKB;
 
-    uint32_t a_bytes, b_bytes = (uint32_t)a.N * (uint32_t)a.ldb * ES;
+    // ---- tile raster: spread over the 8 XCDs so that each XCD's L2 sees a compact block ----
+    auto tile_coords = [&](int pid, int& bz, int& tile_m, int& tile_n, int& tin, int& gsz) {
+        if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+        bz = pid / tiles_mn;
+        const int t = pid - bz * tiles_mn;
+        const int group_sz = a.group_m * a.tiles_n;
+        const int gid = t / group_sz;
+        const int first_m = gid * a.group_m;
+        gsz = min(a.tiles_m - first_m, a.group_m);
+        tin = t - gid * group_sz;
+        tile_m = first_m + tin % gsz;
+        tile_n = tin / gsz;
+    };
+
+    // ---- compute side: the output tile whose accumulators this workgroup holds ----
+    int c_bz, c_tile_m, c_tile_n, c_tin, c_gsz;
+    tile_coords(blockIdx.x, c_bz, c_tile_m, c_tile_n, c_tin, c_gsz);
+    int m0 = c_tile_m * BM, n0 = c_tile_n * BN;
+
+    // ---- issue side: the tile whose k-tiles are being fetched (the same tile unless the launch is persistent) ----
+    uint32_t a_bytes;
+    const uint32_t b_bytes = (uint32_t)a.N * (uint32_t)a.ldb * ES;
     if constexpr (OP == 0) a_bytes = (uint32_t)a.M * (uint32_t)a.lda * ES;
     else a_bytes = (uint32_t)(a.M / (a.HO * a.WO)) * (uint32_t)(a.H * a.W * a.CI) * ES;
-    const rsrc_t rsrcA = make_rsrc(Ab, a_bytes);
-    const rsrc_t rsrcB = make_rsrc(Bb, b_bytes);
+    rsrc_t rsrcA = make_rsrc(a.A, a_bytes);
+    rsrc_t rsrcB = make_rsrc(a.B, b_bytes);
 
-    // ---- per-lane load bookkeeping ----
     const int lrow = lane / CPR, lpos = lane % CPR;
     uint32_t voffB[B_LPW];
-#pragma unroll
-    for (int i = 0; i < B_LPW; ++i) {
-        const int row = (i * NW + wave) * RPI + lrow;
-        const int chunk = lpos ^ swz_of_row(row);
-        const int n = n0 + row;
-        voffB[i] = (n < a.N) ? (uint32_t)n * (uint32_t)a.ldb * ES + chunk * 16 : OOB;
-    }
     // GEMM: byte offset of the lane's chunk in k-tile 0.  Conv: pixel bookkeeping.
     uint32_t voffA[(A_LPW > 0 ? A_LPW : 1)];
     int iy0[OP == 1 ? (A_LPW > 0 ? A_LPW : 1) : 1], ix0[OP == 1 ? (A_LPW > 0 ? A_LPW : 1) : 1];
     int cc = 0, cs = 0, cr = 0;  // conv: channel / kw / kh position of the lane's chunk
-    if constexpr (OP == 0) {
+    int itile = blockIdx.x;
+    int issue_kt = 0;            // next k-tile of tile `itile` to fetch
+
+    auto setup_issue = [&](int t) {
+        const bool alive = t < total;                 // past the last tile every fetch reads zeros
+        int bz, tile_m, tile_n, tin, gsz;
+        tile_coords(alive ? t : 0, bz, tile_m, tile_n, tin, gsz);
+        const int im0 = tile_m * BM, in0 = tile_n * BN;
+        rsrcA = make_rsrc((const char*)a.A + (int64_t)bz * a.sA * ES, a_bytes);
+        rsrcB = make_rsrc((const char*)a.B + (int64_t)bz * a.sB * ES, b_bytes);
 #pragma unroll
-        for (int i = 0; i < A_LPW; ++i) {
+        for (int i = 0; i < B_LPW; ++i) {
             const int row = (i * NW + wave) * RPI + lrow;
             const int chunk = lpos ^ swz_of_row(row);
-            const int m = m0 + row;
-            voffA[i] = (m < a.M) ? (uint32_t)m * (uint32_t)a.lda * ES + chunk * 16 : OOB;
+            const int n = in0 + row;
+            voffB[i] = (alive && n < a.N) ? (uint32_t)n * (uint32_t)a.ldb * ES + chunk * 16 : OOB;
         }
-    } else if constexpr (!CW) {
-        static_assert(OP == 0 || SWZ == 0 || ((NW * RPI) % (CPR << (SWZ > 0 ? SWZ - 1 : 0))) == 0,
-                      "conv: the lane's chunk column must not depend on the load index");
-        const int chunk = lpos ^ swz_of_row(wave * RPI + lrow);
-        int ke = chunk * (16 / ES);                 // element index inside K of tile 0
-        cr = ke / (a.KW * a.CI); ke -= cr * (a.KW * a.CI);
-        cs = ke / a.CI; cc = ke - cs * a.CI;
-        // output pixel of the lane's first row by division, of the following rows (NW*RPI further each) by carry
-        const int hw = a.HO * a.WO;
-        int m = m0 + wave * RPI + lrow;
-        int img = m / hw;
-        int rem = m - img * hw;
-        int oy = rem / a.WO, ox = rem - oy * a.WO;
+        if constexpr (OP == 0) {
 #pragma unroll
-        for (int i = 0; i < A_LPW; ++i) {
-            const bool ok = m < a.M;
-            voffA[i] = (uint32_t)img * (uint32_t)(a.H * a.W * a.CI) * ES;
-            iy0[i] = ok ? oy * a.cstride - a.cpad : -(1 << 28);
-            ix0[i] = ox * a.cstride_w - a.cpad_w;
-            m += NW * RPI;
-            ox += NW * RPI;
-            while (ox >= a.WO) { ox -= a.WO; if (++oy == a.HO) { oy = 0; ++img; } }
+            for (int i = 0; i < A_LPW; ++i) {
+                const int row = (i * NW + wave) * RPI + lrow;
+                const int chunk = lpos ^ swz_of_row(row);
+                const int m = im0 + row;
+                voffA[i] = (alive && m < a.M) ? (uint32_t)m * (uint32_t)a.lda * ES + chunk * 16 : OOB;
+            }
+        } else if constexpr (!CW) {
+            static_assert(OP == 0 || SWZ == 0 || ((NW * RPI) % (CPR << (SWZ > 0 ? SWZ - 1 : 0))) == 0,
+                          "conv: the lane's chunk column must not depend on the load index");
+            const int chunk = lpos ^ swz_of_row(wave * RPI + lrow);
+            int ke = chunk * (16 / ES);                 // element index inside K of tile 0
+            cr = ke / (a.KW * a.CI); ke -= cr * (a.KW * a.CI);
+            cs = ke / a.CI; cc = ke - cs * a.CI;
+            // output pixel of the lane's first row by division, of the following rows (NW*RPI further each) by carry
+            const int hw = a.HO * a.WO;
+            int m = im0 + wave * RPI + lrow;
+            int img = m / hw;
+            int rem = m - img * hw;
+            int oy = rem / a.WO, ox = rem - oy * a.WO;
+#pragma unroll
+            for (int i = 0; i < A_LPW; ++i) {
+                const bool ok = alive && m < a.M;
+                voffA[i] = (uint32_t)img * (uint32_t)(a.H * a.W * a.CI) * ES;
+                iy0[i] = ok ? oy * a.cstride - a.cpad : -(1 << 28);
+                ix0[i] = ox * a.cstride_w - a.cpad_w;
+                m += NW * RPI;
+                ox += NW * RPI;
+                while (ox >= a.WO) { ox -= a.WO; if (++oy == a.HO) { oy = 0; ++img; } }
+            }
         }
-    }
+    };
+    setup_issue(itile);
 
     // L2 prefetch duty of this workgroup.  The tiles that run on one XCD at the same time form a block of
     // a.pf_sb row-tiles x a.pf_sa column-tiles; the pf_sa tiles of one block row read the same rows of A and the
@@ -296,7 +328,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
     if constexpr (PF > 0) {
         constexpr int SEC = BKB >= 64 ? BKB / 64 : 1;
         const int share = pf_isb ? a.pf_sb : a.pf_sa;
-        const int duty = pf_isb ? (tin % gsz) % share : tile_n % share;
+        const int duty = pf_isb ? (c_tin % c_gsz) % share : c_tile_n % share;
         const int q = (pf_isb ? tid - ((NW + 1) / 2) * 64 : tid);      // touch slot inside the operand's waves
         const int row = duty + share * (q / SEC), sec = q % SEC;
         const int g = (pf_isb ? n0 : m0) + row;
@@ -304,7 +336,6 @@ hrn_mfma_kernel(const HrnKArgs a) {
         pf_off[0] = ok ? (uint32_t)g * (uint32_t)(pf_isb ? a.ldb : a.lda) * ES + sec * 64 : OOB;
     }
 
-    int issue_kt = 0;  // next k-tile to fetch
     // Byte offsets of this lane's chunks in k-tile `issue_kt` (out-of-range offset = zeros), shared by both load paths.
     uint32_t offA[(A_LPW > 0 ? A_LPW : 1)], offB[B_LPW];
     auto tile_offsets = [&]() {
@@ -346,6 +377,13 @@ hrn_mfma_kernel(const HrnKArgs a) {
             offB[i] = v;
         }
     };
+    // the stream moves on: next k-tile of this tile, or (persistent) k-tile 0 of the workgroup's next tile
+    auto advance_issue = [&]() {
+        ++issue_kt;
+        if constexpr (PERS) {
+            if (issue_kt == KT) { issue_kt = 0; itile += gridDim.x; setup_issue(itile); }
+        }
+    };
 
     // path 0: fetch k-tile `issue_kt` straight into LDS stage `stage`
     auto issue_tile = [&](int stage) {
@@ -365,7 +403,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
         for (int i = 0; i < A_LPW; ++i) load_chunk_to_lds(rsrcA, sbase + (i * NW + wave) * 1024, offA[i]);
 #pragma unroll
         for (int i = 0; i < B_LPW; ++i) load_chunk_to_lds(rsrcB, sbase + A_BYTES + (i * NW + wave) * 1024, offB[i]);
-        ++issue_kt;
+        advance_issue();
     };
 
     // path 1: fetch k-tile `issue_kt` into register set SET; later copy a set into an LDS stage
@@ -439,16 +477,18 @@ hrn_mfma_kernel(const HrnKArgs a) {
     const int b_lane = A_BYTES + (wn_idx * WTN + lr) * BKB;
 
     acc_t acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < ACC_N; ++r) acc[i][j][r] = 0;
-
     int bsum[TN];
+    auto clear_acc = [&]() {
 #pragma unroll
-    for (int j = 0; j < TN; ++j) bsum[j] = 0;
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < ACC_N; ++r) acc[i][j][r] = 0;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bsum[j] = 0;
+    };
+    clear_acc();
 
     v4i fa[2][TM], fb[2][TN];
     auto read_frags = [&](int buf, int stage_off, int kk) {
@@ -510,6 +550,111 @@ hrn_mfma_kernel(const HrnKArgs a) {
         }
     };
 
+    // ---- epilogue of the compute-side tile (c_bz, m0, n0) ----
+    // MFMA was issued as (B fragment, A fragment), so a lane holds 4 consecutive n for one m:
+    //   m = lr, n = (r/4)*8 + lq*4 + r%4   (32x32)     m = lr, n = lq*4 + r   (16x16)
+    auto store_tile = [&]() {
+        int* bs_lds = (int*)(lds + EPI_OFF);
+        if constexpr (DT == 1) {
+            // 128 * sum_k B[n,k] completes the u8 x s8 product computed as (u8-128) x s8
+            if constexpr (PERS) wait_and_barrier<63, 0>();     // the stages stay live: LDS traffic only, no drain
+            else wait_and_barrier<0, 0>();
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                int s = bsum[j];
+#pragma unroll
+                for (int d = MT; d < 64; d <<= 1) s += __shfl_xor(s, d, 64);
+                if (wm_idx == 0 && lq == 0) bs_lds[wn_idx * WTN + j * MT + lr] = s;
+            }
+            if constexpr (PERS) wait_and_barrier<63, 0>();
+            else __syncthreads();
+        }
+
+        char* Cb = (char*)a.C + (int64_t)c_bz * a.sC * OES;
+        const bool do_store = !(ABL & 16) || a.K == 0x7fffffff;   // the ablation keeps the stores reachable but never takes them
+        if constexpr (EPI == 1) {
+            // LDS-staged epilogue: a wave parks one MFMA row-tile (MT rows x WTN columns) of its result in a private,
+            // padded LDS strip, then streams it out with 16 bytes per lane, whole row segments per store instruction.
+            if constexpr (DT == 0 && !PERS) wait_and_barrier<0, 0>();   // (the int8 path has synchronised above) stages are dead now
+            [[maybe_unused]] const rsrc_t rsrcC = make_rsrc(Cb, (uint32_t)a.M * (uint32_t)a.ldc * OES);
+            char* strip = lds + EPI_OFF + EPI_BASE + wave * (MT * EPI_PITCH);
+            constexpr int CPRW = WTN * OES / 16;               // 16-byte chunks per strip row
+            constexpr int EPC = 16 / OES;                      // output elements per chunk
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                    for (int g = 0; g < ACC_N / 4; ++g) {
+                        const int cl = j * MT + g * 8 + lq * 4;          // column inside the wave tile
+                        char* dst = strip + lr * EPI_PITCH + cl * OES;
+                        if constexpr (DT == 0) {
+                            v4h o;
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[i][j][g * 4 + r];
+                            *(v4h*)dst = o;
+                        } else {
+                            const v4i bs = *(const v4i*)(bs_lds + wn_idx * WTN + cl);
+                            v4i o;
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r] + 128 * bs[r];
+                            *(v4i*)dst = o;
+                        }
+                    }
+                }
+                asm volatile("" ::: "memory");     // LDS serves one wave's requests in order: the reads below see the writes
+#pragma unroll
+                for (int it = 0; it < MT * CPRW / 64; ++it) {
+                    const int c = it * 64 + lane;
+                    const int row = c / CPRW, cc2 = c % CPRW;
+                    const v4i val = *(const v4i*)(strip + row * EPI_PITCH + cc2 * 16);
+                    const int m = m0 + wm_idx * WTM + i * MT + row;
+                    const int n = n0 + wn_idx * WTN + cc2 * EPC;
+                    if constexpr (PERS) {
+                        // always issued, so that every wave has exactly STORES_PER_TILE stores per tile in flight
+                        const uint32_t off = (m < a.M && n + EPC <= a.N) ? (uint32_t)(m * a.ldc + n) * OES : OOB;
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(unsigned int __attribute__((ext_vector_type(4))), val), rsrcC, (int)off, 0, 0);
+                    } else {
+                        char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
+                        if (do_store && m < a.M) {
+                            if (n + EPC <= a.N) *(v4i*)dst = val;
+                            else if (DT == 0 && n + 4 <= a.N) *(long*)dst = ((long)(uint32_t)val.y << 32) | (uint32_t)val.x;
+                        }
+                    }
+                }
+                asm volatile("" ::: "memory");
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int m = m0 + wm_idx * WTM + i * MT + lr;
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                    for (int g = 0; g < ACC_N / 4; ++g) {
+                        const int nl = wn_idx * WTN + j * MT + g * 8 + lq * 4;
+                        const int n = n0 + nl;
+                        if (do_store && m < a.M && n < a.N) {
+                            char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
+                            if constexpr (DT == 0) {
+                                v4h o;
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[i][j][g * 4 + r];
+                                *(v4h*)dst = o;
+                            } else {
+                                const v4i bs = *(const v4i*)(bs_lds + nl);
+                                v4i o;
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r] + 128 * bs[r];
+                                *(v4i*)dst = o;
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    };
+
     if constexpr (LOADM == 0) {
         // ---- prologue: fill all stages, wait for tile 0 ----
     #pragma unroll
@@ -518,30 +663,51 @@ hrn_mfma_kernel(const HrnKArgs a) {
         read_frags(0, 0, 0);
 
         int stage = 0;
-        for (int kt = 0; kt < KT; ++kt) {
-            const int stage_off = stage * STAGE_BYTES;
-            const int next_stage = (stage + 1 == NS) ? 0 : stage + 1;
-            set_masks();
+        auto run_tile = [&](const bool stores_between) {
+            for (int kt = 0; kt < KT; ++kt) {
+                const int stage_off = stage * STAGE_BYTES;
+                const int next_stage = (stage + 1 == NS) ? 0 : stage + 1;
+                set_masks();
     #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) {
-                const int cur = kk & 1;
-                if (kk == KS - 1) {
-                    // every fragment of tile kt is in registers: publish tile kt+1, recycle this stage
-                    if constexpr (ABL & 4) wait_only<(NS - 2) * LPT, 0>();
-                    else wait_and_barrier<(NS - 2) * LPT, 0>();
-                    if (!(ABL & 2)) issue_tile(stage);
-                    advance_reader();
-                    if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, next_stage * STAGE_BYTES, 0);
-                } else {
-                    if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, stage_off, kk + 1);
+                for (int kk = 0; kk < KS; ++kk) {
+                    const int cur = kk & 1;
+                    if (kk == KS - 1) {
+                        // every fragment of tile kt is in registers: publish tile kt+1, recycle this stage
+                        if constexpr (PERS) {
+                            if (stores_between && kt <= NS - 2) wait_and_barrier<(NS - 2) * LPT + STORES_PER_TILE, 0>();
+                            else wait_and_barrier<(NS - 2) * LPT, 0>();
+                        } else if constexpr (ABL & 4) {
+                            wait_only<(NS - 2) * LPT, 0>();
+                        } else {
+                            wait_and_barrier<(NS - 2) * LPT, 0>();
+                        }
+                        if (!(ABL & 2)) issue_tile(stage);
+                        advance_reader();
+                        if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, next_stage * STAGE_BYTES, 0);
+                    } else {
+                        if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, stage_off, kk + 1);
+                    }
+                    if (!(ABL & 8)) mfma_step(cur);
+                    // pin the issue order: fragment reads (and, in the last step, the tile fetch) are
+                    // spread between the MFMAs of this step instead of being sunk behind them
+                    if (kk == KS - 1) sched_pattern<0, TM + TN, TM * TN, LPT>();
+                    else sched_pattern<0, TM + TN, TM * TN, 0>();
                 }
-                if (!(ABL & 8)) mfma_step(cur);
-                // pin the issue order: fragment reads (and, in the last step, the tile fetch) are
-                // spread between the MFMAs of this step instead of being sunk behind them
-                if (kk == KS - 1) sched_pattern<0, TM + TN, TM * TN, LPT>();
-                else sched_pattern<0, TM + TN, TM * TN, 0>();
+                stage = next_stage;
             }
-            stage = next_stage;
+            store_tile();
+        };
+        if constexpr (PERS) {
+            for (int ct = blockIdx.x; ct < total; ct += (int)gridDim.x) {
+                tile_coords(ct, c_bz, c_tile_m, c_tile_n, c_tin, c_gsz);
+                m0 = c_tile_m * BM; n0 = c_tile_n * BN;
+                // the stores of the previous tile's epilogue sit between the fetches that were issued before it and
+                // the ones issued after it; while such a fetch is the one waited for, the wait allows for them
+                run_tile(ct != (int)blockIdx.x && KT >= NS - 1);
+                clear_acc();
+            }
+        } else {
+            run_tile(false);
         }
     } else {
         // ---- register-staged pipeline: tile t is requested during tile t-3's last k-step, copied into LDS
@@ -578,99 +744,6 @@ hrn_mfma_kernel(const HrnKArgs a) {
             body(S0{});
             if (kt + 1 < KT) body(S1{});
         }
-    }
-
-    // ---- epilogue ----
-    // MFMA was issued as (B fragment, A fragment), so a lane holds 4 consecutive n for one m:
-    //   m = lr, n = (r/4)*8 + lq*4 + r%4   (32x32)     m = lr, n = lq*4 + r   (16x16)
-    int* bs_lds = (int*)lds;
-    if constexpr (DT == 1) {
-        // 128 * sum_k B[n,k] completes the u8 x s8 product computed as (u8-128) x s8
-        wait_and_barrier<0, 0>();
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            int s = bsum[j];
-#pragma unroll
-            for (int d = MT; d < 64; d <<= 1) s += __shfl_xor(s, d, 64);
-            if (wm_idx == 0 && lq == 0) bs_lds[wn_idx * WTN + j * MT + lr] = s;
-        }
-        __syncthreads();
-    }
-
-    char* Cb = (char*)a.C + (int64_t)bz * a.sC * OES;
-    const bool do_store = !(ABL & 16) || a.K == 0x7fffffff;   // the ablation keeps the stores reachable but never takes them
-    if constexpr (EPI == 1) {
-        // LDS-staged epilogue: a wave parks one MFMA row-tile (MT rows x WTN columns) of its result in a private,
-        // padded LDS strip, then streams it out with 16 bytes per lane, whole row segments per store instruction.
-        if constexpr (DT == 0) wait_and_barrier<0, 0>();   // (the int8 path has synchronised above) stages are dead now
-        char* strip = lds + EPI_BASE + wave * (MT * EPI_PITCH);
-        constexpr int CPRW = WTN * OES / 16;               // 16-byte chunks per strip row
-        constexpr int EPC = 16 / OES;                      // output elements per chunk
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-#pragma unroll
-                for (int g = 0; g < ACC_N / 4; ++g) {
-                    const int cl = j * MT + g * 8 + lq * 4;          // column inside the wave tile
-                    char* dst = strip + lr * EPI_PITCH + cl * OES;
-                    if constexpr (DT == 0) {
-                        v4h o;
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[i][j][g * 4 + r];
-                        *(v4h*)dst = o;
-                    } else {
-                        const v4i bs = *(const v4i*)(bs_lds + wn_idx * WTN + cl);
-                        v4i o;
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r] + 128 * bs[r];
-                        *(v4i*)dst = o;
-                    }
-                }
-            }
-            asm volatile("" ::: "memory");     // LDS serves one wave's requests in order: the reads below see the writes
-#pragma unroll
-            for (int it = 0; it < MT * CPRW / 64; ++it) {
-                const int c = it * 64 + lane;
-                const int row = c / CPRW, cc = c % CPRW;
-                const v4i val = *(const v4i*)(strip + row * EPI_PITCH + cc * 16);
-                const int m = m0 + wm_idx * WTM + i * MT + row;
-                const int n = n0 + wn_idx * WTN + cc * EPC;
-                char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
-                if (do_store && m < a.M) {
-                    if (n + EPC <= a.N) *(v4i*)dst = val;
-                    else if (DT == 0 && n + 4 <= a.N) *(long*)dst = ((long)(uint32_t)val.y << 32) | (uint32_t)val.x;
-                }
-            }
-            asm volatile("" ::: "memory");
-        }
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int m = m0 + wm_idx * WTM + i * MT + lr;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-#pragma unroll
-            for (int g = 0; g < ACC_N / 4; ++g) {
-                const int nl = wn_idx * WTN + j * MT + g * 8 + lq * 4;
-                const int n = n0 + nl;
-                if (do_store && m < a.M && n < a.N) {
-                    char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
-                    if constexpr (DT == 0) {
-                        v4h o;
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[i][j][g * 4 + r];
-                        *(v4h*)dst = o;
-                    } else {
-                        const v4i bs = *(const v4i*)(bs_lds + nl);
-                        v4i o;
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r] + 128 * bs[r];
-                        *(v4i*)dst = o;
-                    }
-                }
-            }
-        }
+        store_tile();
     }
 }

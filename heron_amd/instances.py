@@ -12,8 +12,8 @@ F16, U8 = B.HRN_DT_F16, B.HRN_DT_U8S8
 GEMM, CONV = B.HRN_OP_GEMM, B.HRN_OP_CONV2D
 
 
-def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, pf=0, load=0, win=0):
-    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, pf, 0, load, win)
+def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, pf=0, load=0, win=0, pers=0):
+    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, pf, 0, load, win, pers)
 
 
 # (bm, bn, bkb, wm, wn, mfma, stages, swizzle): a spread of the template space used by the parity tests
@@ -90,25 +90,46 @@ def int8_conv_descs():
     ]
 
 
+def persistent_descs():
+    """Instances of the persistent (tile-stream) mode in the parity suite: short and long K streams, both element
+    kinds, 2..4 stages, implicit-GEMM conv."""
+    return [
+        D(F16, GEMM, 128, 128, 64, 2, 4, 32, 2, 1, epi=1, pers=1),
+        D(F16, GEMM, 64, 64, 128, 4, 2, 16, 3, 1, epi=1, pers=1),
+        D(F16, GEMM, 256, 128, 128, 4, 2, 32, 2, 2, epi=1, pers=1),
+        D(F16, GEMM, 128, 128, 64, 2, 2, 32, 4, 2, epi=1, pers=1),
+        D(U8, GEMM, 128, 128, 64, 2, 2, 32, 4, 3, epi=1, pers=1),
+        D(U8, GEMM, 64, 128, 256, 1, 2, 16, 2, 1, epi=1, pers=1),
+        D(F16, CONV, 128, 64, 128, 2, 1, 32, 2, 1, epi=1, pers=1),
+        D(U8, CONV, 128, 64, 128, 2, 2, 16, 3, 1, epi=1, pers=1),
+    ]
+
+
+def persistent_twin_descs():
+    """The one-tile-per-workgroup instances with the same tiles as the persistent GEMM instances (bit-identity checks)."""
+    return [D(d.dtype, d.op, *d.as_tuple()[2:10], epi=1) for d in persistent_descs() if d.op == GEMM]
+
+
 # best known instances per benchmark workload (from CGA tuning runs on MI355X); the raster group of
 # each is in BEST_GROUP_M
 BEST = {
     "gemm_f16": D(F16, GEMM, 256, 256, 128, 4, 2, 32, 2, 2, epi=1),
     "gemm_f16_4096": D(F16, GEMM, 256, 256, 128, 2, 4, 32, 2, 2, epi=1, wpe=2),
     "gemm_u8s8": D(U8, GEMM, 256, 256, 64, 2, 4, 32, 4, 3, epi=1),
-    "bmm_f16_qk": D(F16, GEMM, 128, 128, 64, 2, 4, 32, 2, 1, epi=1),
+    "bmm_f16_qk": D(F16, GEMM, 128, 128, 64, 2, 2, 32, 2, 1, epi=1, pers=1),
     "bmm_f16_pv": D(F16, GEMM, 64, 64, 128, 4, 2, 16, 3, 1, epi=1, wpe=1),
     "conv2d_f16": D(F16, CONV, 256, 64, 128, 8, 1, 16, 2, 1, epi=1, win=1),
+    "conv2d_u8s8": D(U8, CONV, 256, 64, 64, 4, 1, 32, 2, 2, epi=1, wpe=2),
     "small": D(U8, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
     "small_f16": D(F16, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
 }
 
-BEST_GROUP_M = {"gemm_f16": 4, "gemm_f16_4096": 4, "gemm_u8s8": 2, "bmm_f16_qk": 8, "bmm_f16_pv": 2, "conv2d_f16": 32}
+BEST_GROUP_M = {"gemm_f16": 4, "gemm_f16_4096": 4, "gemm_u8s8": 2, "bmm_f16_qk": 8, "bmm_f16_pv": 2, "conv2d_f16": 32, "conv2d_u8s8": 32}
 
 
 def all_shipped():
     seen, out = set(), []
-    for d in parity_descs() + variant_descs() + int8_conv_descs() + list(BEST.values()):
+    for d in parity_descs() + variant_descs() + int8_conv_descs() + persistent_descs() + persistent_twin_descs() + list(BEST.values()):
         if d.as_tuple() not in seen:
             seen.add(d.as_tuple())
             out.append(d)

@@ -41,7 +41,12 @@ class Job:
 
 
 def exec(func, queue, args):
-    res = func(*args)
+    try:
+        res = func(*args)
+    except Exception:  # noqa: BLE001 - report the failure at once instead of letting the parent wait for the timeout
+        import traceback
+        traceback.print_exc()
+        res = 0
     queue.put(res)
 
 

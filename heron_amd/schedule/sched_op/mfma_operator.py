@@ -31,7 +31,7 @@ class TemplateSchedule:
         op = B.HRN_OP_CONV2D if self.info['operator'] == 'conv2d_nhwc' else B.HRN_OP_GEMM
         return B.make_desc(dtype, op, p['bm'], p['bn'], p['bkb'], p['wm'], p['wn'], p['mfma'], p['stages'],
                            p['swizzle'], p.get('epilogue', 0), p['waves_per_eu'], p.get('l2_prefetch', 0), 0, 0,
-                           p.get('conv_window', 0))
+                           p.get('conv_window', 0), p.get('persistent', 0))
 
     def to_problem(self):
         from ... import backend as B
@@ -419,6 +419,42 @@ class epilogueOp(schedOp):
         ctx.addSchedDesc("epilogue = %s\n" % s.params['epilogue'])
 
 
+class persistentOp(schedOp):
+    """Launch shape: 0 = one output tile per workgroup, 1 = as many workgroups as the device holds at once, each
+    walking several output tiles with the k-tiles of all of them in one stream through the LDS stages, so the next
+    tile's fetches overlap the current tile's stores.  Needs the LDS-staged epilogue in its own LDS region (the
+    stages stay live), no input window, no L2 prefetch, and the epilogue's store instructions must fit the
+    vector-memory counter together with the fetches issued behind them.  No counterpart in the reference (TVM
+    launches one thread block per output tile)."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        lds_limit = ctx.getLimit('lds_bytes_per_wg')
+        pers = self.knob(ctx, stage_name, 'persistent', [0, 1], 0)
+        km.addLE(pers, self.P(stage_name, 'epilogue'))
+        pw = self.var(ctx, stage_name, 'persistent_plus_window', 0, 1, 0)
+        km.addSUM(pw, [pers, self.P(stage_name, 'conv_window')])
+        if s.info['operator'] == 'gemm':
+            pp = self.var(ctx, stage_name, 'persistent_plus_prefetch', 0, 1, 0)
+            km.addSUM(pp, [pers, self.V(stage_name, 'l2_prefetch_on')])
+        pe = self.var(ctx, stage_name, 'persistent_epi_bytes', 0, lds_limit, 0)
+        km.addProd([pers, self.V(stage_name, 'epi_lds_needed')], pe)
+        tot = self.var(ctx, stage_name, 'lds_bytes_persistent', 2048, lds_limit, 4096)
+        km.addSUM(tot, [self.V(stage_name, 'lds_bytes'), pe])
+        a2 = self.var(ctx, stage_name, 'stages_ahead_minus_1', 0, 3, 0)
+        km.addSUM(self.V(stage_name, 'stages_ahead'), [a2, 1])
+        fl = self.var(ctx, stage_name, 'fetches_behind_stores', 0, 63, 0)
+        km.addProd([a2, self.V(stage_name, 'loads_per_tile')], fl)
+        st = self.var(ctx, stage_name, 'stores_per_tile', 0, 512, 0)
+        km.addProd([self.P(stage_name, 'tile_m'), self.V(stage_name, 'epi_wave_stores')], st)
+        ps = self.var(ctx, stage_name, 'persistent_stores', 0, 63, 0)
+        km.addProd([pers, st], ps)
+        vm = self.var(ctx, stage_name, 'persistent_vmem_in_flight', 0, 63, 0)
+        km.addSUM(vm, [fl, ps])
+        s.params['persistent'] = km.get_val(pers)
+        ctx.addSchedDesc("persistent = %s\n" % s.params['persistent'])
+
+
 class rasterOp(schedOp):
     """Launch-time tile raster: workgroups are spread over the 8 XCDs and walk the tile grid in column
     groups of ``group_m`` row-tiles so that one XCD's L2 holds a compact block of A and B."""
@@ -447,12 +483,13 @@ all_op_methods = {
     'ldsSwizzle': ldsSwizzleOp,
     'registerBudget': registerBudgetOp,
     'epilogue': epilogueOp,
+    'persistent': persistentOp,
     'raster': rasterOp,
     'finish': finishOp,
 }
 
 RULE_ORDER = ['start', 'mfmaShape', 'tileWave', 'tileBlock', 'tileK', 'convWindow', 'loadVector', 'ldsStage', 'ldsSwizzle',
-              'registerBudget', 'epilogue', 'raster', 'finish']
+              'registerBudget', 'epilogue', 'persistent', 'raster', 'finish']
 
 
 def sched_via_rule(ctx, s):

@@ -104,9 +104,13 @@ class Tuner:
         path = self.config.feasible_file_path
         if os.path.exists(path):
             with open(path, 'r') as f:
-                self.feasible = json.loads(f.read())
-            return
+                cached = json.loads(f.read())
+            # a file left by another task or an older constraint set does not cover this task's variables
+            if set(cached.keys()) == set(env.task.knob_manager.solver.vals.keys()):
+                self.feasible = cached
+                return
         print("Feasible not exists, random sample for the first time.")
+        sample_num = getattr(self.config, 'feasible_samples', sample_num)
         population = self.constrained_random_sample(env, int(sample_num), timeout=200)
         dict_set = {}
         for sample in population:

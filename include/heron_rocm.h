@@ -80,6 +80,9 @@ typedef struct hrn_kernel_desc {
     int32_t load_mode;    /* 0 = global -> LDS directly, 1 = global -> registers -> LDS with two tiles in flight (stages must be 2) */
     int32_t conv_window;  /* conv2d only: 1 = keep the reachable input window in LDS and read every filter tap from it
                              (needs stride 1, dilation 1, 'same' padding, CI*2 a multiple of bkb) instead of im2col tiles */
+    int32_t persistent;   /* 1 = launch only as many workgroups as fit the device and let each walk several output tiles,
+                             fetching the next tile's operands while the current result is stored (needs epilogue 1 and
+                             N*out_bytes a multiple of 16) */
 } hrn_kernel_desc;
 
 /* Resource usage of a built instance, for cross-checks of the constraint set. */

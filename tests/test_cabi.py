@@ -26,7 +26,7 @@ def test_header_symbols_exported_and_bound():
 
 
 def test_struct_sizes_match_header_layout():
-    assert ctypes.sizeof(B.KernelDesc) == 16 * 4
+    assert ctypes.sizeof(B.KernelDesc) == 17 * 4
     assert ctypes.sizeof(B.KernelInfo) == 8 * 4
     assert ctypes.sizeof(B.Problem) == 8 * 4 + 3 * 8 + 10 * 4 + 4 * 4
     assert ctypes.sizeof(B.DevInfo) == 64 + 128 + 10 * 4 + 8

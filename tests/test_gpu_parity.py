@@ -237,6 +237,64 @@ def test_conv2d_u8s8_extremes_and_blocked_filter(hrn):
         assert np.array_equal(Y.reshape(ref.shape), ref)
 
 
+PERSIST_GEMM_SHAPES = [(4096, 64, 4096), (1000, 80, 2056), (2048, 528, 512), (96, 4096, 40)]     # (M, K, N), N*out_bytes % 16 == 0
+
+
+@pytest.mark.parametrize("grid", ["", "8", "40"], ids=["device-filling", "8-workgroups", "40-workgroups"])
+@pytest.mark.parametrize("desc", instances.persistent_descs(), ids=lambda d: "-".join(map(str, d.as_tuple())))
+def test_persistent_tile_stream(desc, grid, hrn, monkeypatch):
+    """Persistent instances: every workgroup walks several output tiles and fetches the next tile's operands while the
+    current result is stored.  Few workgroups (8, 40) force many tiles per workgroup, also with short K streams
+    (one or two k-tiles per output tile, i.e. several epilogues inside the fetch window)."""
+    if grid:
+        monkeypatch.setenv("HRN_PERSIST_GRID", grid)
+    else:
+        monkeypatch.delenv("HRN_PERSIST_GRID", raising=False)
+    m = mod_for(desc)
+    f16 = desc.dtype == instances.F16
+    if desc.op == instances.CONV:
+        cases = [(2, 14, 14, 64, 64, 3, 3, 1, 1, 1), (3, 17, 15, 32, 48, 3, 3, 2, 1, 1), (1, 12, 12, 16, 8, 1, 1, 1, 0, 1),
+                 (8, 28, 28, 64, 64, 3, 3, 1, 1, 1)]
+        for i, case in enumerate(cases):
+            N, H, W, CI, CO, KH, KW, s, p, d = case
+            print("persistent conv", desc.as_tuple(), grid, case, flush=True)
+            if f16:
+                X, Wt = workloads.conv2d_inputs(N, H, W, CI, CO, KH, KW, seed=110 + i)
+                check_f16(hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, d).cpu().numpy(), oracle.conv2d_nhwc_f32(X, Wt, s, p, d))
+            else:
+                X, Wt = workloads.conv2d_u8s8_inputs(N, H, W, CI, CO, KH, KW, seed=110 + i)
+                assert np.array_equal(hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, d).cpu().numpy(),
+                                      oracle.conv2d_nhwc_u8s8s32(X, Wt, s, p, d))
+        return
+    for i, (M, K, N) in enumerate(PERSIST_GEMM_SHAPES):
+        print("persistent gemm", desc.as_tuple(), grid, (M, K, N), flush=True)
+        if f16:
+            A, Bm = workloads.gemm_f16_inputs(M, K, N, seed=120 + i)
+            check_f16(hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy(), oracle.gemm_f32(A, Bm))
+        else:
+            A, Bm = workloads.gemm_u8s8_inputs(M, K, N, seed=120 + i)
+            assert np.array_equal(hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy(), oracle.gemm_int64_numpy(A, Bm))
+    # batched, and bit-identical to the one-tile-per-workgroup instance of the same tile (same summation order)
+    t = desc.as_tuple()
+    plain = mod_for(instances.D(desc.dtype, desc.op, *t[2:10], epi=1))
+    if f16:
+        A, Bm = workloads.bmm_qk_inputs(24, 512, 64, 512, seed=7)
+    else:
+        rng = np.random.default_rng(3)
+        A = rng.integers(0, 256, (24, 512, 64), dtype=np.uint8)
+        Bm = rng.integers(-128, 128, (24, 512, 64), dtype=np.int8)
+    C1 = hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy()
+    C0 = hostops.gemm(plain, dev(A), dev(Bm)).cpu().numpy()
+    assert np.array_equal(C1, C0)
+
+
+def test_persistent_rejects_partial_chunks(hrn):
+    m = mod_for(instances.persistent_descs()[0])
+    A, Bm = workloads.gemm_f16_inputs(64, 64, 36, seed=1)              # N*2 is not a multiple of 16
+    with pytest.raises(B.HeronRocmError):
+        hostops.gemm(m, dev(A), dev(Bm))
+
+
 def test_conv_1x1_is_gemm(hrn):
     """A 1x1 convolution is the GEMM of the flattened pixels: both templates must agree bit for bit."""
     tup = instances.PARITY_SHAPES[2]
