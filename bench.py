@@ -100,6 +100,8 @@ MEASURED_TRAFFIC = {
     "gemm_f16_4096": 235.0e6,     # profiles/hrn_mfma_kernel_gemm_f16_4096.md
     "gemm_f16_8192": 1745.9e6,    # profiles/hrn_mfma_kernel_gemm_f16_8192.md
     "gemm_u8s8_8192": 1481.9e6,   # profiles/hrn_mfma_kernel_gemm_u8s8_8192.md
+    "bmm_f16_qk": 126.0e6,        # profiles/hrn_mfma_kernel_conv_bmm.md
+    "conv2d_f16_resnet": 26.5e6,  # profiles/hrn_mfma_kernel_conv_bmm.md
 }
 
 
@@ -235,6 +237,7 @@ def main():
             steps = max(10, min(args.steps, 500))
             wl, e, _ = measure(torch, B, ww, steps, min(args.warmup, 5))
             r = roofline(ww, e, workloads)
+            r["traffic"] = MEASURED_TRAFFIC.get(name)
             also.append({"workload": ww["desc_text"], "value": ww["ops"] / wl / 1e12,
                          "unit": "TFLOP/s" if ww["f16"] else "TOP/s", "kernel_ms": e * 1e3,
                          "frac_of_mfma_peak": ww["ops"] / e / 1e12 / (workloads.PEAK_FP16_TFLOPS if ww["f16"] else workloads.PEAK_INT8_TOPS),
