@@ -1,0 +1,121 @@
+"""The benchmarked instances at the benchmark's full sizes (the shapes `bench.py` times, same tile instance and raster).
+
+A full CPU product of 8192^3 is out of reach for a test, so each result is pinned by
+* the oracle on a random subset of rows / batch entries / images (bit-exact for uint8 x int8, rel. error <= 1e-2 for
+  fp16 inputs with fp32 accumulation), and
+* checksums of checksums that cover EVERY output element: sum_j C[i,j] = A[i,:] . (sum_j B[j,:]) for every row i and
+  sum_i C[i,j] = (sum_i A[i,:]) . B[j,:] for every column j, exact in int64 for the integer path, within the fp16
+  output rounding (2^-11 per element, accumulated as a random walk) for the floating point one.  A single wrong
+  element breaks one row identity and one column identity.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from heron_amd import backend as B
+from heron_amd import hostops, instances, workloads
+
+pytestmark = pytest.mark.gpu
+REL_TOL = 1e-2
+
+
+def dev(a):
+    return torch.from_numpy(a).cuda()
+
+
+def module(key):
+    return B.Module(instances.BEST[key]), instances.BEST_GROUP_M.get(key, 8)
+
+
+def check_rows_f16(C, A, Bm, rows):
+    ref = oracle.gemm_f32(A[rows], Bm)
+    got = C[rows].astype(np.float32)
+    scale = float(np.abs(ref).max())
+    assert float(np.abs(got - ref).max()) / scale <= REL_TOL
+
+
+def check_sums_f16(C, A, Bm):
+    """Row and column checksums in float64 against the closed forms; tolerance = fp16 rounding of the outputs."""
+    C64 = C.astype(np.float64)
+    A64, B64 = A.astype(np.float64), Bm.astype(np.float64)
+    cmax = float(np.abs(C64).max())
+    M, N = C.shape
+    row_ref = A64 @ B64.sum(axis=0)
+    col_ref = A64.sum(axis=0) @ B64.T
+    # each output carries a rounding error <= 2^-11 |C|; a sum of n of them stays within 8 sqrt(n) 2^-11 max|C|
+    assert np.abs(C64.sum(axis=1) - row_ref).max() <= 8 * np.sqrt(N) * 2.0 ** -11 * cmax
+    assert np.abs(C64.sum(axis=0) - col_ref).max() <= 8 * np.sqrt(M) * 2.0 ** -11 * cmax
+
+
+@pytest.mark.parametrize("key,size", [("gemm_f16_4096", 4096), ("gemm_f16", 8192)])
+def test_gemm_f16_full_size(key, size, hrn):
+    m, gm = module(key)
+    A, Bm = workloads.gemm_f16_inputs(size, size, size, seed=1)
+    print("full-size fp16 GEMM", size, instances.BEST[key].as_tuple(), flush=True)
+    C = hostops.gemm(m, dev(A), dev(Bm), group_m=gm).cpu().numpy()
+    rows = np.random.default_rng(0).choice(size, 48, replace=False)
+    check_rows_f16(C, A, Bm, np.sort(rows))
+    check_sums_f16(C, A, Bm)
+
+
+def test_gemm_u8s8_full_size(hrn):
+    m, gm = module("gemm_u8s8")
+    A, Bm = workloads.gemm_u8s8_inputs(8192, 8192, 8192, seed=2)
+    print("full-size u8s8 GEMM", instances.BEST["gemm_u8s8"].as_tuple(), flush=True)
+    C = hostops.gemm(m, dev(A), dev(Bm), group_m=gm).cpu().numpy()
+    rows = np.sort(np.random.default_rng(1).choice(8192, 64, replace=False))
+    assert np.array_equal(C[rows], oracle.gemm_u8s8s32_dlboost(A[rows], Bm))
+    A64, B64 = A.astype(np.int64), Bm.astype(np.int64)
+    assert np.array_equal(C.sum(axis=1, dtype=np.int64), A64 @ B64.sum(axis=0))
+    assert np.array_equal(C.sum(axis=0, dtype=np.int64), A64.sum(axis=0) @ B64.T)
+
+
+@pytest.mark.parametrize("key,gen,shape", [("bmm_f16_qk", workloads.bmm_qk_inputs, (192, 512, 64, 512)),
+                                           ("bmm_f16_pv", workloads.bmm_pv_inputs, (192, 512, 512, 64))])
+def test_bmm_full_size(key, gen, shape, hrn):
+    m, gm = module(key)
+    A, Bm = gen(*shape)
+    print("full-size bmm", key, instances.BEST[key].as_tuple(), flush=True)
+    C = hostops.gemm(m, dev(A), dev(Bm), group_m=gm).cpu().numpy()
+    for b in (0, 1, 95, 190, 191):
+        ref = oracle.gemm_f32(A[b], Bm[b])
+        assert float(np.abs(C[b].astype(np.float32) - ref).max()) / float(np.abs(ref).max()) <= REL_TOL
+    # every batch entry: row checksums against the closed form
+    A64, B64, C64 = A.astype(np.float64), Bm.astype(np.float64), C.astype(np.float64)
+    row_ref = np.einsum("bik,bk->bi", A64, B64.sum(axis=1))
+    tol = 8 * np.sqrt(C.shape[2]) * 2.0 ** -11 * float(np.abs(C64).max())
+    assert np.abs(C64.sum(axis=2) - row_ref).max() <= tol
+    if key == "bmm_f16_pv":
+        # rows of P sum to one, so P.V of a constant V returns that constant (up to fp16 rounding of P)
+        ones = np.ones_like(Bm)
+        R = hostops.gemm(m, dev(A), dev(ones), group_m=gm).cpu().numpy()
+        assert np.abs(R.astype(np.float32) - 1).max() < 5e-3
+
+
+def test_conv2d_f16_full_size(hrn):
+    m, gm = module("conv2d_f16")
+    X, Wt = workloads.conv2d_inputs(32, 56, 56, 64, 64, 3, 3, seed=3)
+    print("full-size fp16 conv", instances.BEST["conv2d_f16"].as_tuple(), flush=True)
+    Y = hostops.conv2d_nhwc(m, dev(X), dev(Wt), 1, 1, 1, group_m=gm).cpu().numpy()
+    for img in (0, 13, 31):
+        ref = oracle.conv2d_nhwc_f32(X[img:img + 1], Wt, 1, 1, 1)
+        assert float(np.abs(Y[img:img + 1].astype(np.float32) - ref).max()) / float(np.abs(ref).max()) <= REL_TOL
+    # every output pixel: the sum over output channels equals the conv with the channel-summed filter
+    Wsum = Wt.astype(np.float32).sum(axis=0, keepdims=True)
+    ref = oracle.conv2d_nhwc_f32(X, Wsum, 1, 1, 1)[..., 0].astype(np.float64)
+    Y64 = Y.astype(np.float64)
+    assert np.abs(Y64.sum(axis=3) - ref).max() <= 8 * np.sqrt(64) * 2.0 ** -11 * float(np.abs(Y64).max())
+
+
+def test_conv2d_u8s8_full_size(hrn):
+    m, gm = module("conv2d_u8s8")
+    X, Wt = workloads.conv2d_u8s8_inputs(32, 56, 56, 64, 64, 3, 3, seed=6)
+    print("full-size u8s8 conv", instances.BEST["conv2d_u8s8"].as_tuple(), flush=True)
+    Y = hostops.conv2d_nhwc(m, dev(X), dev(Wt), 1, 1, 1, group_m=gm).cpu().numpy()
+    for img in (0, 17, 31):
+        assert np.array_equal(Y[img:img + 1], oracle.conv2d_nhwc_u8s8s32(X[img:img + 1], Wt, 1, 1, 1))
+    # every output pixel, exactly: sum over output channels = conv with the channel-summed filter (fits float64 exactly)
+    Wsum = Wt.astype(np.float32).sum(axis=0, keepdims=True)
+    ref = oracle.conv2d_nhwc_f32(X.astype(np.float32), Wsum, 1, 1, 1)[..., 0].astype(np.int64)
+    assert np.array_equal(Y.sum(axis=3, dtype=np.int64), ref)
