@@ -11,6 +11,24 @@ from .conv_variants import (heron_conv1d_ncw, heron_conv1d_nwc, heron_conv2d_nch
 from .reductions import heron_gemv, heron_mean, heron_scan, heron_var
 
 
+class _tolerates_w_format:
+    """The x86 operator set passes the name of its blocked weight layout ("OwI64o4i", "OdhwI64o4i", "OIhw4i16o4i", ...)
+    as the last shape argument (ops/x86/conv1d_int8.py, conv3d_int8.py, dil.py, t2d.py; cases of tests/figure8/configs).
+    The MFMA operators take the filter in the layout their docstring names, so the entry is accepted and dropped.
+    (A class rather than a closure: tasks travel to forked sampler processes and back through pickles.)"""
+
+    def __init__(self, opfunc):
+        self.opfunc = opfunc
+        self.__name__ = opfunc.__name__
+        self.__doc__ = opfunc.__doc__
+
+    def __call__(self, ctx, *args):
+        *shape, in_dtype, out_dtype = args
+        if shape and isinstance(shape[-1], str):
+            shape = shape[:-1]
+        return self.opfunc(ctx, *shape, in_dtype, out_dtype)
+
+
 def getOpFromName(name):
     opmap = {
         "gemm": heron_dense,
@@ -29,4 +47,6 @@ def getOpFromName(name):
         "dil": heron_dil_nhwc,
         "t2d": heron_conv2d_nchw_transposed,
     }
+    if name in ("c1d", "c1d_nwc", "c3d", "c3d_ndhwc", "dil", "t2d", "c2d_nchw"):
+        return _tolerates_w_format(opmap[name])
     return opmap[name]

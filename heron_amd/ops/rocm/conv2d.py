@@ -37,8 +37,8 @@ def heron_conv2d_nhwc(ctx, N, H, W, CI, CO, KH, KW, stride, padding, dilation, *
     if len(dtypes) == 3:
         w_format, in_dtype, out_dtype = dtypes
         assert w_format in W_FORMATS
-        if CO % int(w_format.split('I')[1].split('o')[0]):
-            raise ValueError("CO must be a multiple of the filter block of %s" % w_format)
+        # (the reference floors CO to whole filter blocks, conv2d_int8.py:50,75; the KRSC filter has no blocks, so
+        # every output channel is computed)
     else:
         in_dtype, out_dtype = dtypes
     kind = element_kind(in_dtype)

@@ -163,6 +163,10 @@ class Tuner:
     def constrained_random_sample(self, env, number, timeout=10):
         if self.config.parallel:
             samples = constrained_random_sample_parallel(env.task, number, self.config, timeout)
+            if not samples:
+                # every sampler child failed or timed out: do a smaller batch in this process so the search goes on
+                print("warning: parallel sampling returned nothing, sampling %d points in-process" % min(number, 32))
+                samples = constrained_random_sample_sequential(env.task, min(number, 32), self.config)
         else:
             samples = constrained_random_sample_sequential(env.task, number, self.config)
         perfs = self.predict(samples)

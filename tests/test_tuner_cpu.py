@@ -316,3 +316,35 @@ def test_idea_rank_fronts_and_sa_acceptance():
     assert 0.2 < frac < 0.55                                                         # exp(-0.5/0.5) = 0.37
     assert np.mean([x.predict == 0.5 for x in sa.accept(cur, worse, 0.0)]) == 0      # frozen: never
     assert all(x.predict == 1.0 for x in sa.accept(cur, bad, 0.5))                   # infeasible steps rejected
+
+
+def test_x86_case_forms_with_weight_layout_names_are_accepted():
+    """Cases of the DL Boost experiments carry the blocked weight layout's name as a last shape entry
+    (tests/figure8/configs/c1d.json, c3d.json, dil.json, t2d.json of the reference)."""
+    class Ctx:
+        def set_info(self, info):
+            self.info = info
+
+        def set_axis_map(self, m):
+            pass
+    for name, shape in [("c1d", [1, 892, 512, 1024, 1, 1, 0, 1, 'OwI64o4i']), ("c3d", [1, 8, 56, 56, 64, 64, 3, 3, 3, 1, 1, 1, 'OdhwI64o4i']),
+                        ("dil", [1, 56, 56, 64, 64, 3, 3, 1, 1, 2, 'OhwI64o4i']), ("t2d", [1, 56, 56, 64, 64, 3, 3, 1, 1, 1, 0, 'OIhw4i16o4i']),
+                        ("c2d", [1, 14, 14, 256, 512, 1, 1, 2, 0, 1, 'OhwI48o4i'])]:
+        c = Ctx()
+        out = getOpFromName(name)(c, *shape, "int8", "int32")
+        assert c.info['kind'] == 'u8s8' and out[0].dtype == "int32" and c.info['gemm_view']['K'] % 16 == 0
+
+
+def test_samples_of_every_registry_operator_survive_the_sampler_processes():
+    """Samples are produced in forked children and come back pickled: operator wrappers must not break that."""
+    import pickle
+    from heron_amd.tuner.tuner import constrained_random_sample_parallel
+    cfg = Config()
+    cfg.codegen_type, cfg.parallel_num = 'GPU_MFMA', 2
+    for op, shape in [("c1d", [16, 892, 512, 512, 3, 1, 4, 1]), ("t2d", [16, 14, 14, 64, 32, 4, 4, 2, 1, 1, 0]), ("gemv", [1024, 256])]:
+        t = Task("t", getOpFromName(op), shape + ["float16", "float16"], "rocm")
+        t.config = cfg
+        t.make_stage_schedules()
+        pickle.dumps(t)
+        samples = constrained_random_sample_parallel(t, 4, cfg, 60)
+        assert len(samples) == 4 and all(s.valid for s in samples)
