@@ -36,6 +36,8 @@ class Config:
         self.temperature = 0.6
 
         self.feasible_file_path = 'feasible.json'
+        self.search_generations = 4           # rounds of run_with_pretrained (tuner.py:36; the reference leaves it undefined)
+        self.pretrained_records = []          # records.txt files of earlier tasks for the cross-task cost model
         self.feasible_samples = 1000          # random feasible points behind the per-variable value sets (tuner.py:115)
 
         # defaults for configs created in code rather than from a file

@@ -38,7 +38,15 @@ class Env:
         self.task.make_stage_schedules()
         self.runner.measure_batch = create_measure_batch(self.task, self.runner.measure_option)
         self.dump_schedule()
-        res = self.tuner.run(self)
+        if pretrained or self.config.pretrained_records:
+            from .model import PretrainedCostModel
+            model = PretrainedCostModel(self.task, self.config)
+            n = model.fit_from_records(self.config.pretrained_records, len(self.task.knob_manager.solver.vals))
+            print("pre-trained cost model: %d records from %d files" % (n, len(model.files_used)))
+            self.tuner.setPretrainedModel(model)
+            res = self.tuner.run_with_pretrained(self)
+        else:
+            res = self.tuner.run(self)
         print("Heron tune time spent ", time.time() - start)
         del self.runner.measure_batch
         return res

@@ -41,6 +41,29 @@ class Tuner:
             return res[list(res.keys())[0]]
         return res
 
+    def run_with_pretrained(self, env):
+        """Search steered by a model that was fitted beforehand and is not re-trained (tuner.py:32-45):
+        ``search_generations`` rounds, each measuring the best-predicted max_trials/generations candidates."""
+        self.check_feasible_exits(env)
+        start_time = time.time()
+        gens = max(1, int(self.config.search_generations))
+        population, stat = [], []
+        print("= ---- Tuning with a pre-trained model : Trials %d, Rounds %d ---- =" % (self.config.max_trials, gens))
+        for iter_no in range(gens):
+            print("== Current Round ", iter_no)
+            sample_s = time.time()
+            initial_population = self.UpdatePopulation(env, population, True)
+            population, all_pop = self.optimize(env, initial_population, stat, start_time)
+            sample_e = time.time()
+            pop = self.greedy_select(env, [x for x in all_pop if x.valid], math.ceil(self.config.max_trials / gens))
+            if pop:
+                self.measure(pop, env)
+            with open(os.path.join(self.config.log_dir, 'stat.txt'), 'a') as f:
+                best_perf = env.perf_buffer.best_perf or 0
+                f.write("%d,%f,%f,%f,%f,%f\n" % (iter_no, sample_e - sample_s, time.time() - sample_e, 0.0,
+                                                 time.time() - start_time, best_perf))
+        return population, stat
+
     def run(self, env, do_measure=True):
         self.check_feasible_exits(env)
         start_time = time.time()

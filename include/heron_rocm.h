@@ -90,7 +90,7 @@ typedef struct hrn_kernel_info {
     int32_t vgprs;       /* architectural VGPRs per lane */
     int32_t agprs;       /* accumulation VGPRs per lane */
     int32_t sgprs;
-    int32_t lds_bytes;   /* dynamic LDS the launcher requests */
+    int32_t lds_bytes;   /* static LDS of the kernel; a conv_window instance adds its window at launch */
     int32_t scratch_bytes;
     int32_t occupancy;   /* waves per SIMD the compiler reports */
     int32_t threads;     /* workgroup size */

@@ -103,6 +103,9 @@ if __name__ == '__main__':
     parser.add_argument("-v", "--verbose", action="store_true", help="Show some information if enabled.")
     parser.add_argument("-m", "--max-trials", type=int, default=int(1e6), help="Max trials by command line")
     parser.add_argument("--check", action="store_true", help="verify measured kernels against a host reference")
+    parser.add_argument("--pretrained", type=str, default="",
+                        help="comma separated records.txt files of earlier tasks of the same operator: steer the search "
+                             "with a cost model fitted on them instead of training one from scratch")
     args = parser.parse_args()
     print("Heron device ", args.device_id)
 
@@ -111,6 +114,7 @@ if __name__ == '__main__':
     config.device_id = args.device_id
     config.tuned = args.tuned
     config.verbose = args.verbose
+    config.pretrained_records = [p for p in args.pretrained.split(",") if p]
     runner = HeronRunner.LocalRunner(number=config.runner_number, repeat=config.runner_repeat, min_repeat_ms=0,
                                      timeout=config.runner_timeout, device_id=args.device_id)
     measure_option = HeronRunner.measure_option(

@@ -348,3 +348,25 @@ def test_samples_of_every_registry_operator_survive_the_sampler_processes():
         pickle.dumps(t)
         samples = constrained_random_sample_parallel(t, 4, cfg, 60)
         assert len(samples) == 4 and all(s.valid for s in samples)
+
+
+def test_pretrained_cross_task_model_steers_a_new_task(tmp_path):
+    """Records of one GEMM shape train a model that is used, without re-training, to tune another shape of the same
+    operator (Tuner.run_with_pretrained, tuner/tuner.py:32-45 of the reference)."""
+    env_a = make_env(tmp_path / "a", method="CGA", trials=48)
+    env_a.tune("T1")
+    rec_a = os.path.join(env_a.config.log_dir, "records.txt")
+    env_b = make_env(tmp_path / "b", method="CGA", trials=24, case=("gemm", [2048, 512, 1024]))
+    env_b.config.pretrained_records = [rec_a]
+    env_b.config.search_generations = 2
+    env_b.tune("T1")
+    rows = [json.loads(l) for l in open(os.path.join(env_b.config.log_dir, "records.txt"))]
+    assert 12 <= len(rows) <= 24
+    # the synthetic latency model favours 256x256 tiles; the transferred model finds them within 24 trials
+    assert math.exp(-max(r["perf"] for r in rows)) < 2.0e-3
+    stat = open(os.path.join(env_b.config.log_dir, "stat.txt")).read().strip().splitlines()
+    assert len(stat) == 2
+    # records of another operator family are refused
+    from heron_amd.model import PretrainedCostModel
+    with pytest.raises(ValueError):
+        PretrainedCostModel(env_b.task, env_b.config).fit_from_records([rec_a], 7)
