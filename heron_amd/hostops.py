@@ -163,6 +163,26 @@ def _prep_t2d_nchw(info, X, F):           # (N,CI,H,W), (CO,CI,KH,KW)
     return Xe, _pad_last(F.permute(0, 2, 3, 1), c['CI'])
 
 
+def _prep_dep(info, X, F):                # (N,C,H,W), (K,3,3): the 3x3 windows as 4x4 = 16 taps per pixel and channel
+    d = info['dep']
+    N, C, H, W = X.shape
+    s, p, HO, WO, mult, NP = d['stride'], d['pad'], d['HO'], d['WO'], d['mult'], d['NP']
+    Xp = torch.zeros((N, C, H + 2 * p + 1, W + 2 * p + 1), dtype=X.dtype, device=X.device)
+    Xp[:, :, p:p + H, p:p + W] = X
+    A = torch.zeros((C, N, HO, WO, 4, 4), dtype=X.dtype, device=X.device)
+    for r in range(3):
+        for q in range(3):
+            A[:, :, :, :, r, q] = Xp[:, :, r: r + (HO - 1) * s + 1: s, q: q + (WO - 1) * s + 1: s].permute(1, 0, 2, 3)
+    Bm = torch.zeros((C, NP, 4, 4), dtype=F.dtype, device=F.device)
+    Bm[:, :mult, :3, :3] = F.reshape(C, mult, 3, 3)
+    return A.reshape(C, N * HO * WO, 16), Bm.reshape(C, NP, 16)
+
+
+def _fin_dep(info, Cm):                   # (C, N*HO*WO, NP) -> (N, C, NP, HO, WO)
+    d = info['dep']
+    return Cm.reshape(d['C'], d['N'], d['HO'], d['WO'], d['NP']).permute(1, 0, 4, 2, 3).contiguous()
+
+
 def _fin_identity(info, C):
     return C
 
@@ -201,6 +221,7 @@ ADAPTERS = {
     'c3d_ndhwc': (_prep_c3d_ndhwc, _fin_c3d_ndhwc),
     'c3d_ncdhw': (_prep_c3d_ncdhw, _fin_c3d_ncdhw),
     't2d_nchw': (_prep_t2d_nchw, _fin_nchw),
+    'dep': (_prep_dep, _fin_dep),
 }
 
 

@@ -8,7 +8,7 @@ from .batch_matmul import heron_batch_matmul
 from .conv2d import heron_conv2d_nhwc
 from .conv_variants import (heron_conv1d_ncw, heron_conv1d_nwc, heron_conv2d_nchw, heron_conv2d_nchw_transposed,
                             heron_conv3d_ncdhw, heron_conv3d_ndhwc, heron_dil_nhwc)
-from .reductions import heron_gemv, heron_mean, heron_scan, heron_var
+from .reductions import heron_depthwise_conv2d, heron_gemv, heron_mean, heron_scan, heron_var
 
 
 class _tolerates_w_format:
@@ -46,6 +46,7 @@ def getOpFromName(name):
         "c3d_ndhwc": heron_conv3d_ndhwc,
         "dil": heron_dil_nhwc,
         "t2d": heron_conv2d_nchw_transposed,
+        "dep": heron_depthwise_conv2d,
     }
     if name in ("c1d", "c1d_nwc", "c3d", "c3d_ndhwc", "dil", "t2d", "c2d_nchw"):
         return _tolerates_w_format(opmap[name])

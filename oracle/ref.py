@@ -360,3 +360,22 @@ def conv2d_transposed_nchw_ref(X, F, stride, pad, dil, outpad):
         for s in range(KW):
             out += np.einsum("nchw,oc->nohw", P[:, :, r * dil: r * dil + HO, s * dil: s * dil + WO], _wide(F[:, :, r, s]))
     return out
+
+
+def depthwise_conv2d_ref(X, F, stride, pad):
+    """ops/cuda/dep.py:9-91: X (N,C,H,W), F (K,3,3) with K = mult*C -> (N, C, ceil8(mult), HO, WO);
+    out[n,c,m,p,q] = sum_{r,s<3} Pad(X)[n,c,p*stride+r,q*stride+s] * F[c*mult+m,r,s], rows m >= mult are zero."""
+    N, C, H, W = X.shape
+    K = F.shape[0]
+    mult = K // C
+    NP = (mult + 7) // 8 * 8
+    HO, WO = (H - 3 + 2 * pad) // stride + 1, (W - 3 + 2 * pad) // stride + 1
+    P = np.zeros((N, C, H + 2 * pad, W + 2 * pad), _wide(X).dtype)
+    P[:, :, pad:pad + H, pad:pad + W] = X
+    out = np.zeros((N, C, NP, HO, WO), P.dtype)
+    Fw = _wide(F).reshape(C, mult, 3, 3)
+    for r in range(3):
+        for s in range(3):
+            patch = P[:, :, r: r + (HO - 1) * stride + 1: stride, s: s + (WO - 1) * stride + 1: stride]
+            out[:, :, :mult] += patch[:, :, None] * Fw[None, :, :, r, s, None, None]
+    return out

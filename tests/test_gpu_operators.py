@@ -163,3 +163,14 @@ def test_conv2d_nhwc_height_width_pairs(hrn):
             info, _ = declare("c2d", [N, H, W, CI, CO, KH, KW, s, p, d], dtype)
             ref = oracle.conv2d_nhwc_f32(X, Wt, s, p, d).astype(np.float64) if f16 else oracle.conv2d_nhwc_u8s8s32(X, Wt, s, p, d)
             check(hostops.run_operator(module(info), info, [dev(X), dev(Wt)]), ref, f16)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+def test_depthwise_conv(dtype, hrn):
+    f16 = dtype == "float16"
+    a_dt, b_dt = ("float16", "float16") if f16 else ("uint8", "int8")
+    for (N, H, W, C, K, s, p) in [(2, 14, 14, 32, 32, 1, 1), (1, 17, 15, 24, 48, 2, 1), (2, 9, 9, 16, 48, 1, 0)]:
+        X, F = rnd((N, C, H, W), 17, a_dt), rnd((K, 3, 3), 18, b_dt)
+        print("dep", dtype, (N, H, W, C, K, s, p), flush=True)
+        info, _ = declare("dep", [N, H, W, C, K, 3, 3, s, p, 1], dtype)
+        check(hostops.run_operator(module(info), info, [dev(X), dev(F)]), oracle.depthwise_conv2d_ref(X, F, s, p), f16)

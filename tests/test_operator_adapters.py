@@ -88,3 +88,16 @@ def test_conv3d(s, p, d):
     close(through_adapter("c3d_ndhwc", [2, 6, 9, 7, 5, 12, 3, 3, 2, s, p, d], [X, F]), oracle.conv3d_ndhwc_ref(X, F, s, p, d))
     Xc, Fc = X.transpose(0, 4, 1, 2, 3), F.transpose(4, 3, 0, 1, 2)
     close(through_adapter("c3d", [2, 6, 9, 7, 5, 12, 3, 3, 2, s, p, d], [Xc, Fc]), oracle.conv3d_ncdhw_ref(Xc, Fc, s, p, d))
+
+
+@pytest.mark.parametrize("s,p,mult", [(1, 1, 1), (2, 1, 2)])
+def test_depthwise(s, p, mult):
+    X, F = rnd((2, 6, 9, 8), 16), rnd((6 * mult, 3, 3), 17)
+    c = Ctx()
+    out = getOpFromName("dep")(c, 2, 9, 8, 6, 6 * mult, 3, 3, s, p, 1, "float16", "float16")
+    prep, fin = hostops.ADAPTERS[c.info['adapter']]
+    A, Bm = prep(c.info, torch.from_numpy(X), torch.from_numpy(F))
+    g = c.info['gemm_view']
+    assert tuple(A.shape) == (g['batch'], g['M'], g['K']) and tuple(Bm.shape) == (g['batch'], g['N'], g['K'])
+    C = oracle.bmm_f32(A.numpy(), Bm.numpy())
+    close(fin(c.info, torch.from_numpy(C)).numpy(), oracle.depthwise_conv2d_ref(X, F, s, p))

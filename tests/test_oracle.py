@@ -280,3 +280,13 @@ def test_conv2d_transposed_against_torch(s, p, d, op):
                                                output_padding=op, dilation=d).numpy()
     got = oracle.conv2d_transposed_nchw_ref(X, F, s, p, d, op)
     assert got.shape == ref.shape and np.allclose(got, ref)
+
+
+@pytest.mark.parametrize("s,p,mult", [(1, 1, 1), (2, 1, 2), (1, 0, 3)])
+def test_depthwise_conv_against_torch_grouped_conv(s, p, mult):
+    X, F = _rand((2, 5, 9, 8), 13), _rand((5 * mult, 3, 3), 14)
+    ref = torch.nn.functional.conv2d(torch.from_numpy(X.astype(np.float64)), torch.from_numpy(F.astype(np.float64)).unsqueeze(1),
+                                     stride=s, padding=p, groups=5).numpy()                 # (N, C*mult, HO, WO)
+    got = oracle.depthwise_conv2d_ref(X, F, s, p)
+    assert got.shape[:3] == (2, 5, 8) and not got[:, :, mult:].any()
+    assert np.allclose(got[:, :, :mult].reshape(2, 5 * mult, *got.shape[3:]), ref)

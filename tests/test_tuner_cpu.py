@@ -229,7 +229,8 @@ def test_cost_model_learns_and_ranks():
                                       ("dil", [16, 56, 56, 64, 64, 3, 3, 1, 2, 2]),
                                       ("c3d", [16, 8, 28, 28, 16, 32, 3, 3, 3, 1, 1, 1]),
                                       ("c3d_ndhwc", [16, 8, 28, 28, 16, 32, 3, 3, 3, (2, 1, 1), 1, 1]),
-                                      ("t2d", [16, 14, 14, 64, 32, 4, 4, 2, 1, 1, 0])])
+                                      ("t2d", [16, 14, 14, 64, 32, 4, 4, 2, 1, 1, 0]),
+                                      ("dep", [16, 112, 112, 32, 32, 3, 3, 1, 1, 1])])
 def test_registry_operators_have_a_feasible_template_space(op, shape):
     """Every operator of the registry (ops/cuda/__init__.py:15-32 names) yields a tunable space on the MFMA templates
     whose samples the C side accepts, and announces kernel operands of the GEMM / conv view it declares."""
