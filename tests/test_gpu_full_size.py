@@ -119,3 +119,25 @@ def test_conv2d_u8s8_full_size(hrn):
     Wsum = Wt.astype(np.float32).sum(axis=0, keepdims=True)
     ref = oracle.conv2d_nhwc_f32(X.astype(np.float32), Wsum, 1, 1, 1)[..., 0].astype(np.int64)
     assert np.array_equal(Y.sum(axis=3, dtype=np.int64), ref)
+
+
+def test_largest_operand_the_32_bit_offsets_allow(hrn):
+    """One operand of a batch entry must stay below 2 GiB (buffer offsets are 32-bit): the largest A that fits is
+    multiplied correctly (first, middle and last rows against the oracle), one row more is refused."""
+    m = B.Module(instances.BEST["small_f16"])
+    K, N = 16384, 64
+    M = (2 ** 31 - 1) // (K * 2)                      # 65535 rows: 2 147 450 880 bytes
+    rng = np.random.default_rng(5)
+    Bm = (rng.normal(0, 0.1, (N, K))).astype(np.float16)
+    A = torch.empty((M, K), dtype=torch.float16, device="cuda")
+    A.normal_(0, 0.1)
+    print("largest operand", (M, K, N), flush=True)
+    C = hostops.gemm(m, A, dev(Bm))
+    rows = [0, 1, M // 2, M - 2, M - 1]
+    ref = oracle.gemm_f32(A[rows].cpu().numpy(), Bm)
+    got = C[rows].cpu().numpy().astype(np.float32)
+    assert float(np.abs(got - ref).max()) / float(np.abs(ref).max()) <= REL_TOL
+    del C
+    A2 = torch.empty((M + 1, K), dtype=torch.float16, device="cuda")
+    with pytest.raises(B.HeronRocmError):
+        hostops.gemm(m, A2, dev(Bm))
