@@ -73,8 +73,8 @@ def make_workloads(torch, workloads, instances):
     return W
 
 
-def measure(torch, B, w, steps, warmup):
-    """Returns (wall seconds per step, event seconds per launch)."""
+def measure(torch, B, w, steps, warmup, keep_rows=0):
+    """Returns (wall seconds per step, event seconds per launch, kernel resources[, first rows of the timed output])."""
     mod = B.Module(w["desc"])
     a, b, c, prob = w["build"]()
     stream = torch.cuda.current_stream().cuda_stream
@@ -90,8 +90,9 @@ def measure(torch, B, w, steps, warmup):
     ev = sorted(costs)[len(costs) // 2]
     info = dict(mod.info)
     mod.close()
+    rows = c.reshape(-1, c.shape[-1])[:keep_rows].cpu().numpy() if keep_rows else None
     del a, b, c
-    return wall, ev, info
+    return (wall, ev, info, rows) if keep_rows else (wall, ev, info)
 
 
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
@@ -135,8 +136,9 @@ def roofline(w, ev_seconds, workloads):
             "frac": ach / workloads.PEAK_HBM_GBS, "traffic": None}
 
 
-def cpu_baseline(name, workloads):
-    """The CPU oracle on a bounded sample of the workload (checker code used as a reported baseline only)."""
+def cpu_baseline(name, workloads, gpu_rows=None):
+    """The CPU oracle on a bounded sample of the workload (checker code used as a reported baseline only).  When the
+    first rows of the GPU output of the timed buffers are passed in, the same sample also checks them."""
     import numpy as np
     import oracle
     cores = len(os.sched_getaffinity(0))
@@ -154,9 +156,12 @@ def cpu_baseline(name, workloads):
                 if time.perf_counter() - t0 > 10 or reps >= 20:
                     break
             dt = (time.perf_counter() - t0) / reps
-            return {"value": 2.0 * M * N * K / dt / 1e12, "unit": "TOP/s", "cores": oracle.num_threads(), "kind": "port",
-                    "sample": "full 8192^3 u8s8 GEMM x%d, AVX512-VNNI 16x4 vpdpbusd micro-kernel, B pre-packed, "
-                              "%d OpenMP threads of %d host cores" % (reps, oracle.num_threads(), cores)}
+            out = {"value": 2.0 * M * N * K / dt / 1e12, "unit": "TOP/s", "cores": oracle.num_threads(), "kind": "port",
+                   "sample": "full 8192^3 u8s8 GEMM x%d, AVX512-VNNI 16x4 vpdpbusd micro-kernel, B pre-packed, "
+                             "%d OpenMP threads of %d host cores" % (reps, oracle.num_threads(), cores)}
+            if gpu_rows is not None:
+                out["gpu_rows_bit_exact"] = bool(np.array_equal(gpu_rows, C[:len(gpu_rows)]))
+            return out
         rows = 64
         t0 = time.perf_counter()
         oracle.gemm_u8s8s32_dlboost(A[:rows], Bm)
@@ -177,9 +182,13 @@ def cpu_baseline(name, workloads):
         if time.perf_counter() - t0 > 10 or reps >= 50:
             break
     dt = (time.perf_counter() - t0) / reps
-    return {"value": 2.0 * rows * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
-            "sample": "%d of 4096 rows of the fp16 GEMM 4096^3 x%d, fp32 host reference (double accumulate), "
-                      "%d OpenMP threads of %d host cores" % (rows, reps, oracle.num_threads(), cores)}
+    out = {"value": 2.0 * rows * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+           "sample": "%d of 4096 rows of the fp16 GEMM 4096^3 x%d, fp32 host reference (double accumulate), "
+                     "%d OpenMP threads of %d host cores" % (rows, reps, oracle.num_threads(), cores)}
+    if gpu_rows is not None:
+        ref = oracle.gemm_f32(Af[:len(gpu_rows)], Bf)
+        out["gpu_rows_max_rel_err"] = float(np.abs(gpu_rows.astype(np.float32) - ref).max() / np.abs(ref).max())
+    return out
 
 
 def main():
@@ -212,7 +221,11 @@ def main():
         sys.exit(2)
 
     w = W[args.workload]
-    wall, ev, info = measure(torch, B, w, args.steps, args.warmup)
+    check_rows = 64 if (args.workload in ("gemm_f16_4096", "gemm_u8s8_8192") and not args.only) else 0
+    if check_rows:
+        wall, ev, info, gpu_rows = measure(torch, B, w, args.steps, args.warmup, check_rows)
+    else:
+        (wall, ev, info), gpu_rows = measure(torch, B, w, args.steps, args.warmup), None
     line = {
         "metric": "%s throughput per GPU (tuned MFMA template)" % ("fp16 GEMM TFLOPS" if w["f16"] else "u8s8 GEMM TOPS"),
         "value": w["ops"] / wall / 1e12,
@@ -243,7 +256,7 @@ def main():
                          "frac_of_mfma_peak": ww["ops"] / e / 1e12 / (workloads.PEAK_FP16_TFLOPS if ww["f16"] else workloads.PEAK_INT8_TOPS),
                          "roofline": r})
         line["also"] = also
-        line["cpu_baseline"] = cpu_baseline(args.workload, workloads)
+        line["cpu_baseline"] = cpu_baseline(args.workload, workloads, gpu_rows)
         line["cpu_baseline_u8s8"] = cpu_baseline("gemm_u8s8_8192", workloads) if not args.workload.startswith("gemm_u8s8") else None
     print(json.dumps(line))
 
