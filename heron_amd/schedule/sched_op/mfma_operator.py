@@ -210,7 +210,7 @@ class convWindowOp(schedOp):
                   c['HO'] == c['H'] and c['WO'] == c['W'] and c['KH'] * c['KW'] <= 32)
             pitch = c['CI'] * (2 if s.info['kind'] == 'f16' else 1)
             halo = 2 * (c['pad'] * c['W'] + c['pad_w'])
-        win = self.knob(ctx, stage_name, 'conv_window', [0, 1] if ok else [0], 1 if ok else 0)
+        win = self.knob(ctx, stage_name, 'conv_window', [0, 1] if ok else [0], 0)
         staged = self.var(ctx, stage_name, 'a_rows_staged', 0, 512, 16)       # rows of A that go through the stages
         off = self.var(ctx, stage_name, 'conv_window_off', 0, 1, 1)
         km.addSUM(1, [win, off])

@@ -46,7 +46,10 @@ class Task:
             json_dict = json.loads(row)
             to_sort.append((json_dict['perf'], json_dict['param']))
         sorted_pairs = sorted(to_sort, key=lambda x: -x[0])
-        self.knob_manager.solved_knob_vals_phenotype = sorted_pairs[0][1]
+        # a record written before a knob was added to the template lacks that knob: it then takes its default (off)
+        param = {name: var.defv for name, var in self.knob_manager.solver.vals.items()}
+        param.update(sorted_pairs[0][1])
+        self.knob_manager.solved_knob_vals_phenotype = param
         self.knob_manager.runtime_perf = sorted_pairs[0][0]
         self.knob_manager.is_building = False
         return self.instantiate(self.knob_manager)

@@ -1,0 +1,51 @@
+"""Writes fuzz_instances.json: template instances drawn from the tuner's own search space (constrained random
+samples of the CDNA4 constraint set, fixed seed), so that the GPU parity suite also covers knob combinations nobody
+picked by hand.  build() compiles them with the other shipped instances.
+
+usage: python tests/golden/make_fuzz_instances.py
+"""
+import copy
+import json
+import os
+import random
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.abspath(os.path.join(HERE, "..", "..")))
+
+import numpy as np                                                    # noqa: E402
+
+from heron_amd import backend as B                                    # noqa: E402
+from heron_amd.config import Config                                   # noqa: E402
+from heron_amd.ops.rocm import getOpFromName                          # noqa: E402
+from heron_amd.task.task import Task                                  # noqa: E402
+
+TASKS = [("gemm", [2048, 1024, 2048], "float16", 8), ("gemm", [2048, 1024, 2048], "int8", 8),
+         ("bmm", [8, 512, 256, 512], "float16", 4), ("c2d", [4, 28, 28, 64, 128, 3, 3, 1, 1, 1], "float16", 8),
+         ("c2d", [4, 28, 28, 64, 128, 3, 3, 1, 1, 1], "int8", 6), ("c2d", [2, 30, 30, 32, 64, 3, 3, 2, 1, 1], "float16", 4)]
+
+if __name__ == "__main__":
+    random.seed(20240607)
+    np.random.seed(20240607)
+    out, seen = [], set()
+    for op, shape, dtype, count in TASKS:
+        cfg = Config()
+        cfg.codegen_type = 'GPU_MFMA'
+        t = Task("t", getOpFromName(op), shape + [dtype, dtype], "rocm")
+        t.config = cfg
+        t.make_stage_schedules()
+        got = 0
+        while got < count:
+            km = copy.deepcopy(t.knob_manager)
+            valid, _ = km.randSample({})
+            s, _ = t.instantiate(km)
+            d = s.to_desc()
+            tup = d.as_tuple()
+            if not valid or not B.check_desc(d) or tup in seen:
+                continue
+            seen.add(tup)
+            out.append({"desc": list(tup), "group_m": int(s.params["group_m"]), "from": [op, shape, dtype]})
+            got += 1
+    with open(os.path.join(HERE, "fuzz_instances.json"), "w") as f:
+        json.dump(out, f, indent=0)
+    print(len(out), "instances")
