@@ -132,6 +132,7 @@ SYMBOLS = {
     "hrn_launch_conv2d_nhwc_u8s8": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
     "hrn_launch_repeat": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _vp]),
     "hrn_time": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _i, _d, ctypes.POINTER(_d), _vp]),
+    "hrn_time_cold": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_problem_gemm": (None, [ctypes.POINTER(Problem), _i, _i, _i, _i]),
     "hrn_problem_conv2d": (None, [ctypes.POINTER(Problem)] + [_i] * 10),
     "hrn_problem_conv2d_hw": (None, [ctypes.POINTER(Problem)] + [_i] * 13),
@@ -249,6 +250,13 @@ class Module:
     def launch_repeat(self, problem, a_ptr, b_ptr, c_ptr, count, stream=0):
         """``count`` back-to-back launches issued from one host call."""
         _check(lib().hrn_launch_repeat(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, count, stream))
+
+    def time_cold(self, problem, a_ptr, b_ptr, c_ptr, flush_ptr, flush_bytes, repeat=4, stream=0):
+        """Seconds of ``repeat`` single launches, each after the caches were flushed with the caller's buffer."""
+        costs = (_d * repeat)()
+        _check(lib().hrn_time_cold(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, flush_ptr, flush_bytes, repeat,
+                                   costs, stream))
+        return list(costs)
 
     def time(self, problem, a_ptr, b_ptr, c_ptr, number=3, repeat=4, min_repeat_ms=0.0, stream=0):
         costs = (_d * repeat)()

@@ -733,6 +733,42 @@ int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const v
     return HRN_OK;
 }
 
+int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* flush_buf,
+                  size_t flush_bytes, int repeat, double* costs_out, void* stream) {
+    if (!costs_out || repeat < 1 || !flush_buf || flush_bytes < (64u << 20)) return fail(HRN_E_BADPARAM, "repeat/costs_out/flush buffer (>= 64 MiB)");
+    HrnKArgs k;
+    unsigned grid;
+    unsigned dyn_lds;
+    int rc = fill_args(mod, p, A, B, C, &k, &grid, &dyn_lds);
+    if (rc) return rc;
+    int dev = 0;
+    hipDeviceProp_t pr;
+    HIP_TRY(hipGetDevice(&dev));
+    HIP_TRY(hipGetDeviceProperties(&pr, dev));
+    hipStream_t st = (hipStream_t)stream;
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    auto cleanup = [&]() { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); };
+    rc = launch(mod, p, A, B, C, stream);  // surfaces launch errors before anything is timed
+    if (rc) { cleanup(); return rc; }
+    const size_t half16 = flush_bytes / 32;   // 16-byte elements in each half of the flush buffer
+    for (int r = 0; r < repeat; ++r) {
+        // stream one half of the flush buffer into the other: every L2 and the memory-side cache are refilled with it
+        probe_copy_kernel<<<pr.multiProcessorCount * 16, 256, 0, st>>>((const pv4i*)flush_buf, (pv4i*)flush_buf + half16, half16);
+        (void)hipEventRecord(e0, st);
+        rc = launch(mod, p, A, B, C, stream);
+        if (rc) { cleanup(); return rc; }
+        (void)hipEventRecord(e1, st);
+        if (hipEventSynchronize(e1) != hipSuccess) { cleanup(); return fail(HRN_E_LAUNCH, "kernel failed: %s", hipGetErrorString(hipGetLastError())); }
+        float ms = 0;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        costs_out[r] = (double)ms * 1e-3;
+    }
+    cleanup();
+    return HRN_OK;
+}
+
 void hrn_problem_gemm(hrn_problem* p, int batch, int m, int n, int k) {
     memset(p, 0, sizeof *p);
     p->op = HRN_OP_GEMM;

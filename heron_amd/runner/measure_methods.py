@@ -117,6 +117,7 @@ def _server_main(conn, device_id):
         from .. import backend as B
         torch.cuda.set_device(device_id)
         mods = {}
+        flush = None
         conn.send(("ready", None))
     except Exception:  # noqa: BLE001
         conn.send(("error", traceback.format_exc()))
@@ -133,7 +134,8 @@ def _server_main(conn, device_id):
             if kind == "info":
                 conn.send(("ok", B.device_info(device_id)))
                 continue
-            _, desc_tuple, prob, arg_info, number, repeat, min_repeat_ms, ref_input, ref_output, rtol = req
+            _, desc_tuple, prob, arg_info, number, repeat, min_repeat_ms, ref_input, ref_output, rtol = req[:10]
+            cold = len(req) > 10 and req[10]
             if desc_tuple not in mods:
                 if len(mods) > 64:
                     mods.pop(next(iter(mods))).close()
@@ -157,8 +159,15 @@ def _server_main(conn, device_id):
                     t = torch.randint(-128, 128, shape, dtype=tdt, device="cuda")
                 tensors.append(t)
             torch.cuda.synchronize()
-            costs = mod.time(p, tensors[0].data_ptr(), tensors[1].data_ptr(), tensors[-1].data_ptr(),
-                             number, repeat, min_repeat_ms, 0)
+            if cold:
+                # every launch starts from flushed caches (the reference runner's enable_cpu_cache_flush, on the GPU)
+                if flush is None:
+                    flush = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+                costs = mod.time_cold(p, tensors[0].data_ptr(), tensors[1].data_ptr(), tensors[-1].data_ptr(),
+                                      flush.data_ptr(), flush.numel(), repeat, 0)
+            else:
+                costs = mod.time(p, tensors[0].data_ptr(), tensors[1].data_ptr(), tensors[-1].data_ptr(),
+                                 number, repeat, min_repeat_ms, 0)
             errno = MeasureErrorNo.NO_ERROR
             if ref_output is not None:
                 out = tensors[-1].cpu().numpy()
@@ -178,6 +187,7 @@ class HipRunner:
         self.min_repeat_ms = min_repeat_ms
         self.timeout = timeout
         self.cooldown_interval = cooldown_interval
+        self.cache_flush = bool(enable_cpu_cache_flush)
         self.device_id = device_id
         self.task = None
         self._proc = None
@@ -256,7 +266,7 @@ class HipRunner:
             verify = not task.not_verify_correctness
             req = ("measure", br.desc_tuple, br.problem, br.arg_info, self.number, self.repeat,
                    float(self.min_repeat_ms), task.ref_input if verify else None,
-                   task.ref_output if verify else None, getattr(task, "rtol", 0.1))
+                   task.ref_output if verify else None, getattr(task, "rtol", 0.1), self.cache_flush)
             status, payload = self._request(req, self.timeout)
             tstamp = time.time()
             if status == "ok":
@@ -274,13 +284,13 @@ class HipRunner:
                 time.sleep(self.cooldown_interval)
         return results
 
-    def time_instance(self, s, args, number=3, repeat=4, min_repeat_ms=500):
+    def time_instance(self, s, args, number=3, repeat=4, min_repeat_ms=500, cold=False):
         """Final timing of one instance, as tests/quick_start/*/run.py:52-62 of the reference does with
         time_evaluator; returns the mean seconds per launch."""
         from .. import backend as B
         B.compile_desc(s.to_desc(), 300.0)
         req = ("measure", s.to_desc().as_tuple(), _problem_to_dict(s.to_problem()),
-               [(tuple(t.shape), t.dtype) for t in args], number, repeat, float(min_repeat_ms), None, None, 0.1)
+               [(tuple(t.shape), t.dtype) for t in args], number, repeat, float(min_repeat_ms), None, None, 0.1, cold)
         status, payload = self._request(req, max(self.timeout, 120))
         if status != "ok":
             raise RuntimeError("timing failed: %s %s" % (status, payload))

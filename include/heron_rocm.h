@@ -182,6 +182,15 @@ int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const v
              int number, int repeat, double min_repeat_ms, double* costs_out, void* stream);
 
 /*
+ * Cold-cache variant: before each of the `repeat` single launches, `flush_bytes` of caller-owned device memory at
+ * flush_buf (use at least twice the last-level cache: 1 GiB covers the 256 MiB memory-side cache) are streamed through
+ * the caches, so the launch finds its operands in HBM only.  The GPU-side counterpart of the reference runner's
+ * `enable_cpu_cache_flush` (tests/quick_start/dlboost/run.py:89-96, runner/measure_methods.py:138-145).
+ */
+int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C,
+                  void* flush_buf, size_t flush_bytes, int repeat, double* costs_out, void* stream);
+
+/*
  * Roofline probes (no counterpart in the reference, which never relates a timing to a hardware
  * limit).  hrn_probe_mfma times a register-resident loop of independent MFMAs of the given
  * dtype/shape on every CU and returns dense T(FL)OP/s (random_operands != 0 feeds operands with the

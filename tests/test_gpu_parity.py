@@ -378,3 +378,21 @@ def test_device_info_and_timing(hrn):
                    min_repeat_ms=1.0)
     assert len(costs) == 4 and all(0 < x < 1e-2 for x in costs)
     check_f16(c.cpu().numpy(), oracle.gemm_f32(A, Bm))
+
+
+def test_cold_cache_timing(hrn):
+    """Launches timed after a cache flush: the 4 MiB-operand GEMM that lives in L2/MALL when repeated takes longer
+    from HBM, and the result is still correct."""
+    m = mod_for(instances.BEST["gemm_f16_4096"])
+    A, Bm = workloads.gemm_f16_inputs(2048, 1024, 2048, seed=4)
+    a, b = dev(A), dev(Bm)
+    c = torch.empty((2048, 2048), dtype=torch.float16, device="cuda")
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    p = B.gemm_problem(1, 2048, 2048, 1024, 4)
+    warm = sorted(m.time(p, a.data_ptr(), b.data_ptr(), c.data_ptr(), number=20, repeat=5))[2]
+    cold = sorted(m.time_cold(p, a.data_ptr(), b.data_ptr(), c.data_ptr(), flush.data_ptr(), flush.numel(), repeat=5))[2]
+    print("warm %.2f us, cold %.2f us" % (warm * 1e6, cold * 1e6), flush=True)
+    assert 0 < warm < cold < 100 * warm
+    check_f16(c.cpu().numpy(), oracle.gemm_f32(A, Bm))
+    with pytest.raises(B.HeronRocmError):
+        m.time_cold(p, a.data_ptr(), b.data_ptr(), c.data_ptr(), flush.data_ptr(), 1024, repeat=2)
