@@ -247,7 +247,11 @@ int compile_desc(const hrn_kernel_desc* d, double timeout_s, std::string* out_pa
     if (!file_exists(src)) return fail(HRN_E_BUILD, "kernel template not found: %s", src.c_str());
     const std::string dir = cache_dir();
     mkdir(dir.c_str(), 0755);
-    const std::string key = desc_key(d, fnv1a_file(src));
+    // extra compiler flags (e.g. -D switches of the template under study) are part of the instance's identity
+    const std::string extra = env_or("HRN_HIPCC_FLAGS", "");
+    uint64_t srch = fnv1a_file(src);
+    for (unsigned char ch : extra) { srch ^= ch; srch *= 1099511628211ull; }
+    const std::string key = desc_key(d, srch);
     const std::string co = dir + "/" + key + ".hsaco";
     const std::string info = dir + "/" + key + ".info";
     *out_path = co;
@@ -270,6 +274,11 @@ int compile_desc(const hrn_kernel_desc* d, double timeout_s, std::string* out_pa
     def("HRN_LOAD", d->load_mode);
     def("HRN_CONVWIN", d->conv_window);
     def("HRN_PERSIST", d->persistent);
+    {
+        std::stringstream es(extra);
+        std::string tok;
+        while (es >> tok) args.push_back(tok);
+    }
     args.push_back(src);
     args.push_back("-o");
     args.push_back(co_tmp);
