@@ -69,6 +69,19 @@ int fail(int code, const char* fmt, ...) {
         if (e_ != hipSuccess) return fail(HRN_E_LAUNCH, "%s: %s", #expr, hipGetErrorString(e_)); \
     } while (0)
 
+// two timing events that are destroyed on every exit path
+struct EventPair {
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t create() {
+        hipError_t e = hipEventCreate(&e0);
+        return e != hipSuccess ? e : hipEventCreate(&e1);
+    }
+    ~EventPair() {
+        if (e0) (void)hipEventDestroy(e0);
+        if (e1) (void)hipEventDestroy(e1);
+    }
+};
+
 std::string lib_dir() {
     Dl_info di;
     if (dladdr((void*)&hrn_last_error, &di) && di.dli_fname) {
@@ -506,9 +519,9 @@ int hrn_probe_mfma(int dtype, int mfma, int random_operands, double* tops_out, v
     hipStream_t st = (hipStream_t)stream;
     const int iters = 20000, grid = pr.multiProcessorCount * 2;   // 2 workgroups x 4 waves per CU: 2 waves per SIMD
     const int kind = (dtype == HRN_DT_F16 ? 0 : 2) + (mfma == 32 ? 0 : 1);
-    hipEvent_t e0, e1;
-    HIP_TRY(hipEventCreate(&e0));
-    HIP_TRY(hipEventCreate(&e1));
+    EventPair ev;
+    HIP_TRY(ev.create());
+    hipEvent_t e0 = ev.e0, e1 = ev.e1;
     float ms = 0;
     for (int rep = 0; rep < 2; ++rep) {   // first pass warms up
         (void)hipEventRecord(e0, st);
@@ -520,11 +533,9 @@ int hrn_probe_mfma(int dtype, int mfma, int random_operands, double* tops_out, v
         }
         (void)hipEventRecord(e1, st);
         hipError_t e = hipEventSynchronize(e1);
-        if (e != hipSuccess) { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); return fail(HRN_E_LAUNCH, "probe: %s", hipGetErrorString(e)); }
+        if (e != hipSuccess) return fail(HRN_E_LAUNCH, "probe: %s", hipGetErrorString(e));
         (void)hipEventElapsedTime(&ms, e0, e1);
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
     const double ops_per_mfma = (dtype == HRN_DT_F16) ? 32768.0 : 65536.0;   // 2*m*n*k for either shape
     const double total = ops_per_mfma * (mfma == 32 ? 1.0 : 0.5) * 4.0 * iters * 4.0 * grid;  // 4 accumulators, 4 waves
     *tops_out = total / (ms * 1e-3) / 1e12;
@@ -538,9 +549,9 @@ int hrn_probe_copy(const void* src, void* dst, size_t bytes, int repeat, double*
     hipDeviceProp_t pr;
     HIP_TRY(hipGetDeviceProperties(&pr, dev));
     hipStream_t st = (hipStream_t)stream;
-    hipEvent_t e0, e1;
-    HIP_TRY(hipEventCreate(&e0));
-    HIP_TRY(hipEventCreate(&e1));
+    EventPair ev;
+    HIP_TRY(ev.create());
+    hipEvent_t e0 = ev.e0, e1 = ev.e1;
     const int grid = pr.multiProcessorCount * 16;
     probe_copy_kernel<<<grid, 256, 0, st>>>((const pv4i*)src, (pv4i*)dst, bytes / 16);
     (void)hipEventRecord(e0, st);
@@ -549,8 +560,6 @@ int hrn_probe_copy(const void* src, void* dst, size_t bytes, int repeat, double*
     hipError_t e = hipEventSynchronize(e1);
     float ms = 0;
     (void)hipEventElapsedTime(&ms, e0, e1);
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
     if (e != hipSuccess) return fail(HRN_E_LAUNCH, "probe: %s", hipGetErrorString(e));
     *gbs_out = 2.0 * bytes * repeat / (ms * 1e-3) / 1e9;
     return HRN_OK;
@@ -709,23 +718,22 @@ int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const v
     int rc = fill_args(mod, p, A, B, C, &k, &grid, &dyn_lds);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
-    hipEvent_t e0, e1;
-    HIP_TRY(hipEventCreate(&e0));
-    HIP_TRY(hipEventCreate(&e1));
-    auto cleanup = [&]() { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); };
+    EventPair ev;
+    HIP_TRY(ev.create());
+    hipEvent_t e0 = ev.e0, e1 = ev.e1;
     rc = launch(mod, p, A, B, C, stream);  // warm-up, also surfaces launch errors
-    if (rc) { cleanup(); return rc; }
-    if (hipStreamSynchronize(st) != hipSuccess) { cleanup(); return fail(HRN_E_LAUNCH, "warm-up failed: %s", hipGetErrorString(hipGetLastError())); }
+    if (rc) return rc;
+    if (hipStreamSynchronize(st) != hipSuccess) { return fail(HRN_E_LAUNCH, "warm-up failed: %s", hipGetErrorString(hipGetLastError())); }
     for (int r = 0; r < repeat; ++r) {
         int num = number;
         for (;;) {
             (void)hipEventRecord(e0, st);
             for (int i = 0; i < num; ++i) {
                 rc = launch(mod, p, A, B, C, stream);
-                if (rc) { cleanup(); return rc; }
+                if (rc) return rc;
             }
             (void)hipEventRecord(e1, st);
-            if (hipEventSynchronize(e1) != hipSuccess) { cleanup(); return fail(HRN_E_LAUNCH, "kernel failed: %s", hipGetErrorString(hipGetLastError())); }
+            if (hipEventSynchronize(e1) != hipSuccess) { return fail(HRN_E_LAUNCH, "kernel failed: %s", hipGetErrorString(hipGetLastError())); }
             float ms = 0;
             (void)hipEventElapsedTime(&ms, e0, e1);
             if (ms >= min_repeat_ms || num >= (1 << 20)) {
@@ -738,7 +746,6 @@ int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const v
             num = std::max(num + 1, (int)std::min(1048576.0, min_repeat_ms * 1.2 / per + 1));
         }
     }
-    cleanup();
     return HRN_OK;
 }
 
@@ -755,26 +762,24 @@ int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, co
     HIP_TRY(hipGetDevice(&dev));
     HIP_TRY(hipGetDeviceProperties(&pr, dev));
     hipStream_t st = (hipStream_t)stream;
-    hipEvent_t e0, e1;
-    HIP_TRY(hipEventCreate(&e0));
-    HIP_TRY(hipEventCreate(&e1));
-    auto cleanup = [&]() { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); };
+    EventPair ev;
+    HIP_TRY(ev.create());
+    hipEvent_t e0 = ev.e0, e1 = ev.e1;
     rc = launch(mod, p, A, B, C, stream);  // surfaces launch errors before anything is timed
-    if (rc) { cleanup(); return rc; }
+    if (rc) return rc;
     const size_t half16 = flush_bytes / 32;   // 16-byte elements in each half of the flush buffer
     for (int r = 0; r < repeat; ++r) {
         // stream one half of the flush buffer into the other: every L2 and the memory-side cache are refilled with it
         probe_copy_kernel<<<pr.multiProcessorCount * 16, 256, 0, st>>>((const pv4i*)flush_buf, (pv4i*)flush_buf + half16, half16);
         (void)hipEventRecord(e0, st);
         rc = launch(mod, p, A, B, C, stream);
-        if (rc) { cleanup(); return rc; }
+        if (rc) return rc;
         (void)hipEventRecord(e1, st);
-        if (hipEventSynchronize(e1) != hipSuccess) { cleanup(); return fail(HRN_E_LAUNCH, "kernel failed: %s", hipGetErrorString(hipGetLastError())); }
+        if (hipEventSynchronize(e1) != hipSuccess) { return fail(HRN_E_LAUNCH, "kernel failed: %s", hipGetErrorString(hipGetLastError())); }
         float ms = 0;
         (void)hipEventElapsedTime(&ms, e0, e1);
         costs_out[r] = (double)ms * 1e-3;
     }
-    cleanup();
     return HRN_OK;
 }
 

@@ -15,7 +15,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-def convert(src, max_trials=128):
+def convert(src, max_trials=256):
     c = json.load(open(src))["config"]
     cases = {}
     for key, (op, shape, count) in c["cases"].items():
