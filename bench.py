@@ -276,8 +276,13 @@ def main():
                          "frac_of_mfma_peak": ww["ops"] / e / 1e12 / (workloads.PEAK_FP16_TFLOPS if ww["f16"] else workloads.PEAK_INT8_TOPS),
                          "roofline": r})
         line["also"] = also
-        line["cpu_baseline"] = cpu_baseline(args.workload, workloads, gpu_rows)
-        line["cpu_baseline_u8s8"] = cpu_baseline("gemm_u8s8_8192", workloads) if not args.workload.startswith("gemm_u8s8") else None
+        def guarded(*a):
+            try:
+                return cpu_baseline(*a)
+            except Exception as e:  # noqa: BLE001 - the GPU figures above are still worth printing
+                return {"value": None, "unit": None, "cores": 0, "kind": "port", "sample": "failed: %r" % (e,)}
+        line["cpu_baseline"] = guarded(args.workload, workloads, gpu_rows)
+        line["cpu_baseline_u8s8"] = guarded("gemm_u8s8_8192", workloads) if not args.workload.startswith("gemm_u8s8") else None
     print(json.dumps(line))
 
 
