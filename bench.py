@@ -106,6 +106,13 @@ MEASURED_TRAFFIC = {
 }
 
 
+def safe_probes(torch, B):
+    try:
+        return run_probes(torch, B)
+    except Exception as e:  # noqa: BLE001 - context figures only
+        return {"error": repr(e)[:200]}
+
+
 def run_probes(torch, B):
     """Roofline denominators measured on this GPU next to the published ones."""
     n = 1 << 30
@@ -261,18 +268,22 @@ def main():
     line["roofline"]["traffic"] = MEASURED_TRAFFIC.get(args.workload)
     line["peaks"] = {"published": {"mfma_f16_TFLOPs": workloads.PEAK_FP16_TFLOPS, "mfma_i8_TOPs": workloads.PEAK_INT8_TOPS,
                                    "hbm_GBs": workloads.PEAK_HBM_GBS},
-                     "measured": run_probes(torch, B), "used": "published"}
+                     "measured": safe_probes(torch, B), "used": "published"}
     if not args.only:
         also = []
         for name, ww in W.items():
             if name == args.workload:
                 continue
             steps = max(10, min(args.steps, 500))
-            wl, e, _ = measure(torch, B, ww, steps, min(args.warmup, 5))
+            try:
+                wl, e, _ = measure(torch, B, ww, steps, min(args.warmup, 5))
+            except Exception as err:  # noqa: BLE001 - one side workload must not cost the headline
+                also.append({"workload": ww["desc_text"], "error": repr(err)[:200]})
+                continue
             r = roofline(ww, e, workloads)
             r["traffic"] = MEASURED_TRAFFIC.get(name)
             also.append({"workload": ww["desc_text"], "value": ww["ops"] / wl / 1e12,
-                         "unit": "TFLOP/s" if ww["f16"] else "TOP/s", "kernel_ms": e * 1e3,
+                         "unit": "TFLOP/s" if ww["f16"] else "TOP/s", "steps": steps, "kernel_ms": e * 1e3,
                          "frac_of_mfma_peak": ww["ops"] / e / 1e12 / (workloads.PEAK_FP16_TFLOPS if ww["f16"] else workloads.PEAK_INT8_TOPS),
                          "roofline": r})
         line["also"] = also
