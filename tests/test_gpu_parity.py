@@ -396,3 +396,44 @@ def test_cold_cache_timing(hrn):
     check_f16(c.cpu().numpy(), oracle.gemm_f32(A, Bm))
     with pytest.raises(B.HeronRocmError):
         m.time_cold(p, a.data_ptr(), b.data_ptr(), c.data_ptr(), flush.data_ptr(), 1024, repeat=2)
+
+
+def test_launches_from_several_host_threads(hrn):
+    """Four host threads launch through the same library at once, each on a stream of its own: two share one module,
+    two have their own.  Every result must match what the oracle gives for that thread's inputs."""
+    import threading
+    shared = mod_for(instances.BEST["small_f16"])
+    mods = [shared, shared, mod_for(instances.BEST["small"]), mod_for(instances.D(instances.F16, instances.GEMM, *instances.PARITY_SHAPES[0]))]
+    shapes = [(192, 128, 320), (130, 72, 64), (256, 144, 96), (64, 264, 200)]
+    inputs, outs, errors = [], [None] * 4, []
+    for i, (m, (M, K, N)) in enumerate(zip(mods, shapes)):
+        gen = workloads.gemm_f16_inputs if m.desc.dtype == B.HRN_DT_F16 else workloads.gemm_u8s8_inputs
+        A, Bm = gen(M, K, N, seed=70 + i)
+        inputs.append((A, Bm, dev(A), dev(Bm)))
+    torch.cuda.synchronize()
+    start = threading.Barrier(4)
+
+    def work(i):
+        try:
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                start.wait()
+                for _ in range(50):
+                    out = hostops.gemm(mods[i], inputs[i][2], inputs[i][3])
+                s.synchronize()
+            outs[i] = out.cpu().numpy()
+        except Exception as e:       # reported by the main thread
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(60)
+    assert not errors, errors
+    for i, m in enumerate(mods):
+        A, Bm = inputs[i][0], inputs[i][1]
+        if m.desc.dtype == B.HRN_DT_F16:
+            check_f16(outs[i], oracle.gemm_f32(A, Bm))
+        else:
+            assert np.array_equal(outs[i], oracle.gemm_int64_numpy(A, Bm).astype(np.int32))
