@@ -185,8 +185,8 @@ def lds_bytes(desc):
 
 def compile_desc(desc, timeout_s=0.0):
     """hipcc the instance into the cache (no GPU needed); returns the code object path."""
-    buf = ctypes.create_string_buffer(1024)
-    _check(lib().hrn_compile(ctypes.byref(desc), float(timeout_s), buf, 1024))
+    buf = ctypes.create_string_buffer(4096)
+    _check(lib().hrn_compile(ctypes.byref(desc), float(timeout_s), buf, 4096))
     return buf.value.decode()
 
 

@@ -604,7 +604,11 @@ int hrn_compile(const hrn_kernel_desc* desc, double timeout_s, char* path_out, s
     std::string path;
     int rc = compile_desc(desc, timeout_s, &path);
     if (rc) return rc;
-    if (path_out && path_cap) snprintf(path_out, path_cap, "%s", path.c_str());
+    if (path_out) {
+        if (path.size() + 1 > path_cap)
+            return fail(HRN_E_BADPARAM, "path buffer of %zu bytes is too small for %zu", path_cap, path.size() + 1);
+        memcpy(path_out, path.c_str(), path.size() + 1);
+    }
     return HRN_OK;
 }
 

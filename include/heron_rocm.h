@@ -134,7 +134,8 @@ int hrn_check_desc(const hrn_kernel_desc* desc);
  * Compiles one template instance with hipcc into the on-disk cache and returns the path of
  * the code object.  Touches no GPU (safe in forked/pooled builder processes).  Stands in for
  * autotvm.LocalBuilder -> tvm.build (tests/quick_start/dlboost/run.py:89-96), including its
- * `build_timeout` (config.py:48): timeout_s <= 0 means no limit.
+ * `build_timeout` (config.py:48): timeout_s <= 0 means no limit.  path_out may be NULL; a buffer
+ * that cannot hold the path and its terminator is HRN_E_BADPARAM.
  */
 int hrn_compile(const hrn_kernel_desc* desc, double timeout_s, char* path_out, size_t path_cap);
 

@@ -63,3 +63,25 @@ def test_compile_without_gpu_and_shipped_instances_present():
     path = B.compile_desc(d, 120.0)
     assert path.endswith(".hsaco") and os.path.getsize(path) > 1000
     assert os.path.exists(path[:-6] + ".info")
+
+
+def test_compile_error_paths(tmp_path, monkeypatch):
+    """A path buffer that is too small, a compiler that fails and a compiler that outlives the limit are reported as
+    errors with a message; nothing is left in the cache for them."""
+    import stat
+    d = instances.BEST["small"]
+    L = B.lib()
+    tiny = ctypes.create_string_buffer(8)
+    assert L.hrn_compile(ctypes.byref(d), 120.0, tiny, 8) == -1 and b"too small" in L.hrn_last_error()
+    assert L.hrn_compile(ctypes.byref(d), 120.0, None, 0) == 0
+    monkeypatch.setenv("HRN_CACHE_DIR", str(tmp_path / "cache"))
+    monkeypatch.setenv("HRN_HIPCC_FLAGS", "--no-such-flag")
+    buf = ctypes.create_string_buffer(4096)
+    assert L.hrn_compile(ctypes.byref(d), 120.0, buf, 4096) == -2 and b"hipcc failed" in L.hrn_last_error()
+    monkeypatch.setenv("HRN_HIPCC_FLAGS", "")
+    slow = tmp_path / "slow_cc.sh"
+    slow.write_text("#!/bin/sh\nsleep 30\n")
+    slow.chmod(slow.stat().st_mode | stat.S_IEXEC)
+    monkeypatch.setenv("HRN_HIPCC", str(slow))
+    assert L.hrn_compile(ctypes.byref(d), 0.5, buf, 4096) == -5 and b"exceeded" in L.hrn_last_error()
+    assert not list((tmp_path / "cache").glob("*.hsaco"))
