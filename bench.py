@@ -103,6 +103,8 @@ MEASURED_TRAFFIC = {
     "gemm_u8s8_8192": 1481.9e6,   # profiles/hrn_mfma_kernel_gemm_u8s8_8192.md
     "bmm_f16_qk": 126.0e6,        # profiles/hrn_mfma_kernel_conv_bmm.md
     "conv2d_f16_resnet": 26.5e6,  # profiles/hrn_mfma_kernel_conv_bmm.md
+    "bmm_f16_pv": 125.9e6,        # profiles/hrn_mfma_kernel_conv_bmm.md
+    "conv2d_u8s8_resnet": 32.6e6, # profiles/hrn_mfma_kernel_conv_bmm.md
 }
 
 
