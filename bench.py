@@ -99,8 +99,8 @@ def measure(torch, B, w, steps, warmup, keep_rows=0):
 # what the same counters read for the plain copy kernel of known size (profiles/ holds the runs these come from)
 MEASURED_TRAFFIC = {
     "gemm_f16_4096": 235.0e6,     # profiles/hrn_mfma_kernel_gemm_f16_4096.md
-    "gemm_f16_8192": 1745.9e6,    # profiles/hrn_mfma_kernel_gemm_f16_8192.md
-    "gemm_u8s8_8192": 1481.9e6,   # profiles/hrn_mfma_kernel_gemm_u8s8_8192.md
+    "gemm_f16_8192": 1746.1e6,    # profiles/hrn_mfma_kernel_gemm_f16_8192.md
+    "gemm_u8s8_8192": 1074.4e6,   # profiles/hrn_mfma_kernel_gemm_u8s8_8192.md
     "bmm_f16_qk": 126.0e6,        # profiles/hrn_mfma_kernel_conv_bmm.md
     "conv2d_f16_resnet": 26.5e6,  # profiles/hrn_mfma_kernel_conv_bmm.md
     "bmm_f16_pv": 125.9e6,        # profiles/hrn_mfma_kernel_conv_bmm.md

@@ -26,12 +26,14 @@ PARITY_SHAPES = [
     (128, 128, 128, 2, 2, 16, 2, 1),
     (64, 128, 256, 1, 2, 16, 2, 1),
     (32, 32, 128, 1, 2, 16, 4, 0),
+    (256, 256, 128, 2, 4, 16, 2, 2),
 ]
 
 
 # instances that exercise the optional load paths: (tile tuple, l2_prefetch, load_mode)
 # (tile tuple) instances run with the LDS-staged epilogue as well
 EPILOGUE_VARIANTS = [
+    (256, 256, 128, 2, 4, 16, 2, 2),
     (256, 256, 128, 4, 2, 32, 2, 2),
     (256, 256, 64, 2, 4, 32, 4, 3),
     (128, 128, 128, 2, 2, 32, 2, 1),
@@ -97,6 +99,7 @@ def persistent_descs():
         D(F16, GEMM, 128, 128, 64, 2, 4, 32, 2, 1, epi=1, pers=1),
         D(F16, GEMM, 64, 64, 128, 4, 2, 16, 3, 1, epi=1, pers=1),
         D(F16, GEMM, 256, 128, 128, 4, 2, 32, 2, 2, epi=1, pers=1),
+        D(F16, GEMM, 256, 128, 128, 4, 2, 16, 2, 2, epi=1, pers=1),
         D(F16, GEMM, 128, 128, 64, 2, 2, 32, 4, 2, epi=1, pers=1),
         D(U8, GEMM, 128, 128, 64, 2, 2, 32, 4, 3, epi=1, pers=1),
         D(U8, GEMM, 64, 128, 256, 1, 2, 16, 2, 1, epi=1, pers=1),
@@ -113,10 +116,10 @@ def persistent_twin_descs():
 # best known instances per benchmark workload (from CGA tuning runs on MI355X); the raster group of
 # each is in BEST_GROUP_M
 BEST = {
-    "gemm_f16": D(F16, GEMM, 256, 256, 128, 4, 2, 32, 2, 2, epi=1),
-    "gemm_f16_4096": D(F16, GEMM, 256, 256, 128, 2, 4, 32, 2, 2, epi=1, wpe=2),
-    "gemm_u8s8": D(U8, GEMM, 256, 256, 64, 2, 4, 32, 4, 3, epi=1),
-    "bmm_f16_qk": D(F16, GEMM, 128, 128, 64, 2, 2, 32, 2, 1, epi=1, pers=1),
+    "gemm_f16": D(F16, GEMM, 256, 256, 128, 2, 4, 16, 2, 2, epi=1),
+    "gemm_f16_4096": D(F16, GEMM, 256, 256, 128, 2, 4, 16, 2, 2, epi=1),
+    "gemm_u8s8": D(U8, GEMM, 256, 256, 128, 2, 4, 16, 2, 2, epi=1),
+    "bmm_f16_qk": D(F16, GEMM, 256, 128, 128, 4, 2, 16, 2, 2, epi=1, pers=1),
     "bmm_f16_pv": D(F16, GEMM, 64, 64, 128, 4, 2, 16, 3, 1, epi=1, wpe=1),
     "conv2d_f16": D(F16, CONV, 512, 64, 128, 8, 1, 32, 2, 1, epi=1, wpe=1, win=1),
     "conv2d_u8s8": D(U8, CONV, 256, 64, 64, 4, 1, 32, 2, 2, epi=1, wpe=2, win=1),
@@ -124,7 +127,7 @@ BEST = {
     "small_f16": D(F16, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
 }
 
-BEST_GROUP_M = {"gemm_f16": 4, "gemm_f16_4096": 4, "gemm_u8s8": 2, "bmm_f16_qk": 8, "bmm_f16_pv": 2, "conv2d_f16": 32, "conv2d_u8s8": 32}
+BEST_GROUP_M = {"gemm_f16": 4, "gemm_f16_4096": 4, "gemm_u8s8": 4, "bmm_f16_qk": 8, "bmm_f16_pv": 2, "conv2d_f16": 32, "conv2d_u8s8": 32}
 
 
 def all_shipped():

@@ -332,12 +332,16 @@ class ldsSwizzleOp(schedOp):
 
 
 class registerBudgetOp(schedOp):
-    """Register file: accumulators tm*tn*(mfma^2/64) <= 256 per lane, plus double-buffered operand
-    fragments 8*(tm+tn) and a fixed allowance for addresses; times the waves each SIMD hosts
-    (waves/4, at least 1) it must fit the 512-entry unified VGPR+AGPR file.  No counterpart in the
-    reference (NVCC allocates registers behind TVM's back)."""
+    """Register file: accumulators tm*tn*(mfma^2/64) <= 256 per lane, plus operand fragments and a fixed
+    allowance for addresses; times the waves each SIMD hosts (waves/4, at least 1) it must fit the
+    512-entry unified VGPR+AGPR file.  The fragment term 6*(tm+tn) and the allowance are fitted to what
+    hipcc allocates for compiled instances (it keeps less than two full fragment sets live): 256x256
+    tiles on 8 waves take 200 registers with 32x32 MFMAs (tm+tn = 6) and 226-247 with 16x16 MFMAs
+    (tm+tn = 12), both of which must stay in the space.  No counterpart in the reference (NVCC
+    allocates registers behind TVM's back)."""
 
-    OVERHEAD = 48
+    OVERHEAD = 32
+    FRAG_REGS = 6
 
     def perform(self, s, stage_name, ctx):
         km = ctx.knob_manager
@@ -350,8 +354,8 @@ class registerBudgetOp(schedOp):
         km.addProd([tmn, self.V(stage_name, 'acc_regs_per_tile')], acc)
         tsum = self.var(ctx, stage_name, 'tile_m_plus_n', 2, 32, 4)
         km.addSUM(tsum, [tm, tn])
-        frag = self.var(ctx, stage_name, 'frag_regs', 16, 256, 32)
-        km.addProd([8, tsum], frag)
+        frag = self.var(ctx, stage_name, 'frag_regs', 6, 256, 36)
+        km.addProd([self.FRAG_REGS, tsum], frag)
         regs = self.var(ctx, stage_name, 'regs_per_lane', 1, regs_total, 128)
         km.addSUM(regs, [acc, frag, self.OVERHEAD])
         # waves of one workgroup that share a SIMD
