@@ -113,7 +113,7 @@ def persistent_twin_descs():
     return [D(d.dtype, d.op, *d.as_tuple()[2:10], epi=1) for d in persistent_descs() if d.op == GEMM]
 
 
-# best known instances per benchmark workload (from CGA tuning runs on MI355X); the raster group of
+# best known instances per benchmark workload (from CGA tuning runs on MI355X and sweeps around their results); the raster group of
 # each is in BEST_GROUP_M
 BEST = {
     "gemm_f16": D(F16, GEMM, 256, 256, 128, 2, 4, 16, 2, 2, epi=1),
