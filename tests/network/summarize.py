@@ -1,6 +1,7 @@
 """Tables of the network-level results:  python summarize.py            rewrites results/README.md from results/*.json
                                        python summarize.py --merge NET NEW.json RECORDS_DIR
-                                           folds a later run of ``run.py -c configs/NET.json -o NEW.json`` into
+                                           folds a later run of ``run.py -c configs/NET.json -o NEW.json`` (or, with
+                                           ``-`` for NEW.json, the best search measurements in RECORDS_DIR) into
                                            results/NET.json, keeping the faster instance per layer, and copies the best
                                            record of every layer that improved from RECORDS_DIR/<layer>/records.txt into
                                            tuned/NET/<layer>/records.txt (what ``run.py -T tuned/NET`` re-times).
@@ -52,7 +53,18 @@ def best_record(path):
 
 def merge(net, new_json, records_dir):
     old_path = os.path.join(HERE, "results", net + ".json")
-    old, new = json.load(open(old_path)), json.load(open(new_json))
+    old = json.load(open(old_path))
+    if new_json == "-":
+        # an interrupted run leaves no table: take the best measurement of the search from each layer's records
+        new = dict(max_trials=0, layers=[])
+        for case in sorted(os.listdir(records_dir)):
+            recs = [json.loads(line) for line in open(os.path.join(records_dir, case, "records.txt"))]
+            good = [r["latency"] for r in recs if r["perf"] > 0]
+            if good:
+                new["layers"].append(dict(case=case, latency_ms=min(good) * 1e3))
+                new["max_trials"] = max(new["max_trials"], len(recs))
+    else:
+        new = json.load(open(new_json))
     by_case = {r["case"]: r for r in new["layers"]}
     for r in old["layers"]:
         r.setdefault("trials", old["max_trials"])
