@@ -149,6 +149,41 @@ def run_probes(torch, B):
             del a, b
     except Exception as e:  # noqa: BLE001
         out["vendor_library_error"] = repr(e)[:200]
+    # the library's int8 product (signed x signed -> int32, the closest it offers to the u8 x s8 GEMM) on random bytes
+    try:
+        n = 8192
+        a = torch.randint(-128, 128, (n, n), device="cuda", dtype=torch.int8)
+        b = torch.randint(-128, 128, (n, n), device="cuda", dtype=torch.int8)
+        for _ in range(5):
+            torch._int_mm(a, b.t())
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(50):
+            torch._int_mm(a, b.t())
+        e1.record()
+        torch.cuda.synchronize()
+        out["vendor_library_gemm_s8s8_8192_TOPs"] = 2.0 * n ** 3 / (e0.elapsed_time(e1) * 1e-3 / 50) / 1e12
+        del a, b
+    except Exception as e:  # noqa: BLE001
+        out["vendor_library_int8_error"] = repr(e)[:200]
+    # the library's convolution (torch conv2d = MIOpen) on the ResNet-50 stage-2 shape, channels-last fp16 in and out
+    try:
+        x = torch.relu(torch.randn(32, 64, 56, 56, device="cuda")).half().contiguous(memory_format=torch.channels_last)
+        w = (torch.randn(64, 64, 3, 3, device="cuda") * 0.05).half().contiguous(memory_format=torch.channels_last)
+        for _ in range(5):
+            torch.nn.functional.conv2d(x, w, padding=1)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(500):
+            torch.nn.functional.conv2d(x, w, padding=1)
+        e1.record()
+        torch.cuda.synchronize()
+        out["vendor_library_conv2d_f16_resnet_us"] = e0.elapsed_time(e1) * 1e3 / 500
+        del x, w
+    except Exception as e:  # noqa: BLE001
+        out["vendor_library_conv_error"] = repr(e)[:200]
     return out
 
 
