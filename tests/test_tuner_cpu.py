@@ -372,3 +372,32 @@ def test_pretrained_cross_task_model_steers_a_new_task(tmp_path):
     from heron_amd.model import PretrainedCostModel
     with pytest.raises(ValueError):
         PretrainedCostModel(env_b.task, env_b.config).fit_from_records([rec_a], 7)
+
+
+TUNED = os.path.join(os.path.dirname(os.path.abspath(__file__)), "quick_start", "rocm", "tuned")
+
+
+@pytest.mark.parametrize("rel,op,shape,dtype", [
+    ("GEMM_F16_4096/G4096", "gemm", [4096, 4096, 4096], "float16"),
+    ("GEMM_F16_8192/G8192", "gemm", [8192, 8192, 8192], "float16"),
+    ("GEMM_INT8/G8192", "gemm", [8192, 8192, 8192], "int8"),
+    ("C2D_F16/C1", "c2d", [32, 56, 56, 64, 64, 3, 3, 1, 1, 1], "float16"),
+    ("C2D_INT8/C1", "c2d", [32, 56, 56, 64, 64, 3, 3, 1, 1, 1, "OhwI64o4i"], "int8")])
+def test_shipped_tuned_records_reinstantiate(rel, op, shape, dtype):
+    """The records kept for ``run.py -t`` (the 32 best of a search on MI355X per benchmark case) are feasible points of
+    today's constraint system and Task.apply_best turns the best of them into a template instance the library accepts."""
+    path = os.path.join(TUNED, rel, "records.txt")
+    rows = [json.loads(l) for l in open(path)]
+    assert 1 <= len(rows) <= 32 and all(r["perf"] > 0 for r in rows)
+    cfg = Config()
+    cfg.codegen_type = 'GPU_MFMA'
+    t = Task("t", getOpFromName(op), shape + [dtype, dtype], "rocm")
+    t.config = cfg
+    t.make_stage_schedules()
+    for r in rows:
+        assert t.knob_manager.solver.SATScore(dict(r["param"])) == 0
+    s, args = t.apply_best(path)
+    assert B.check_desc(s.to_desc()), B.lib().hrn_last_error()
+    best = max(rows, key=lambda r: r["perf"])
+    stage = s.info['stage_name']
+    assert s.params['bm'] == best["param"]["V#ST:%s,AX:None,VA:block_m" % stage]
