@@ -121,13 +121,13 @@ BEST = {
     "gemm_u8s8": D(U8, GEMM, 256, 256, 128, 2, 4, 16, 2, 2, epi=1),
     "bmm_f16_qk": D(F16, GEMM, 256, 128, 128, 4, 2, 16, 2, 2, epi=1, pers=1),
     "bmm_f16_pv": D(F16, GEMM, 64, 64, 128, 4, 2, 16, 3, 1, epi=1, wpe=1),
-    "conv2d_f16": D(F16, CONV, 512, 64, 128, 8, 1, 32, 2, 1, epi=1, wpe=1, win=1),
+    "conv2d_f16": D(F16, CONV, 512, 64, 128, 8, 1, 32, 2, 2, epi=1, win=1),
     "conv2d_u8s8": D(U8, CONV, 256, 64, 64, 4, 1, 32, 2, 2, epi=1, wpe=2, win=1),
     "small": D(U8, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
     "small_f16": D(F16, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
 }
 
-BEST_GROUP_M = {"gemm_f16": 4, "gemm_f16_4096": 4, "gemm_u8s8": 4, "bmm_f16_qk": 8, "bmm_f16_pv": 2, "conv2d_f16": 32, "conv2d_u8s8": 32}
+BEST_GROUP_M = {"gemm_f16": 4, "gemm_f16_4096": 4, "gemm_u8s8": 4, "bmm_f16_qk": 8, "bmm_f16_pv": 2, "conv2d_f16": 16, "conv2d_u8s8": 32}
 
 
 def all_shipped():
