@@ -171,16 +171,19 @@ def run_probes(torch, B):
     try:
         x = torch.relu(torch.randn(32, 64, 56, 56, device="cuda")).half().contiguous(memory_format=torch.channels_last)
         w = (torch.randn(64, 64, 3, 3, device="cuda") * 0.05).half().contiguous(memory_format=torch.channels_last)
+        for _ in range(20):            # the library's first calls of a shape run a slow fallback kernel
+            torch.nn.functional.conv2d(x, w, padding=1)
+        torch.cuda.synchronize()
+        groups = []
         for _ in range(5):
-            torch.nn.functional.conv2d(x, w, padding=1)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(500):
-            torch.nn.functional.conv2d(x, w, padding=1)
-        e1.record()
-        torch.cuda.synchronize()
-        out["vendor_library_conv2d_f16_resnet_us"] = e0.elapsed_time(e1) * 1e3 / 500
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(100):
+                torch.nn.functional.conv2d(x, w, padding=1)
+            e1.record()
+            torch.cuda.synchronize()
+            groups.append(e0.elapsed_time(e1) * 1e3 / 100)
+        out["vendor_library_conv2d_f16_resnet_us"] = min(groups)
         del x, w
     except Exception as e:  # noqa: BLE001
         out["vendor_library_conv_error"] = repr(e)[:200]
