@@ -381,6 +381,8 @@ TUNED = os.path.join(os.path.dirname(os.path.abspath(__file__)), "quick_start", 
     ("GEMM_F16_4096/G4096", "gemm", [4096, 4096, 4096], "float16"),
     ("GEMM_F16_8192/G8192", "gemm", [8192, 8192, 8192], "float16"),
     ("GEMM_INT8/G8192", "gemm", [8192, 8192, 8192], "int8"),
+    ("BMM_F16/QK", "bmm", [192, 512, 64, 512], "float16"),
+    ("BMM_F16/PV", "bmm", [192, 512, 512, 64], "float16"),
     ("C2D_F16/C1", "c2d", [32, 56, 56, 64, 64, 3, 3, 1, 1, 1], "float16"),
     ("C2D_INT8/C1", "c2d", [32, 56, 56, 64, 64, 3, 3, 1, 1, 1, "OhwI64o4i"], "int8")])
 def test_shipped_tuned_records_reinstantiate(rel, op, shape, dtype):
