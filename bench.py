@@ -2,13 +2,20 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
-One step = one launch of the tuned template instance over a batch of synthetic operands that are
-already resident in HBM.  Prints ONE JSON line.  The headline workload is the dense fp16 GEMM
-M=N=K=4096 (fp32 accumulate, fp16 output); the other benchmark configurations are reported under
-"also" in the same line.  `roofline.achieved` is algorithmic work per launch divided by the average
-kernel duration measured with HIP events on the launch stream.  `cpu_baseline` times the CPU oracle
-(the DL Boost-style VNNI GEMM for the quantized case, the fp32 host reference otherwise) on a bounded
-sample of the same workload, on this machine's host cores.
+One step = one launch of the tuned template instance over a batch of synthetic operands that are already resident in
+HBM.  Prints ONE JSON line.  The headline workload is the quantized GEMM M=N=K=8192 (uint8 x int8 -> int32); the other
+benchmark configurations are reported under "also" in the same line.  Every instance is the best record of
+tests/quick_start/rocm/tuned/<case>/records.txt, replayed through Task.apply_best.
+
+Timing.  Before anything is timed the same kernel runs untimed until the chip's clocks have settled (at least 200 ms,
+then until two consecutive 20-launch groups agree within 2 %); this does not depend on --warmup.  Then --warmup untimed
+launches, then exactly --steps launches bracketed by torch.cuda.synchronize() for ``value`` / ``ms_per_step`` and by
+HIP events on the launch stream for ``config.kernel_ms`` (what ``roofline.achieved`` is computed from).  Rows bounded by
+HBM are also timed cold - every launch after 1 GiB was streamed through the caches - and their roofline fraction
+is the cold one: back-to-back launches of a 126 MB problem run out of the 256 MB memory-side cache.
+
+``cpu_baseline`` times the CPU oracle's DL Boost-style GEMM (AVX512-VNNI 16x4 micro-kernel, all host cores) on the
+same 8192^3 problem and checks the first rows of the very buffer that was timed against it.
 """
 import argparse
 import json
@@ -20,9 +27,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+HEADLINE = "gemm_u8s8_8192"
 
-def make_workloads(torch, workloads, instances):
-    """name -> dict(desc, problem factory, device operands, ops, bytes, peak, dtype)."""
+
+def make_workloads(torch, workloads, tuned):
+    """name -> dict(instance, problem factory, ops, bytes, f16, text)."""
     from heron_amd import backend as B
 
     def dev(a):
@@ -30,8 +39,8 @@ def make_workloads(torch, workloads, instances):
 
     W = {}
 
-    def add_gemm(name, key, M, K, N, f16, batch=1, gen=None):
-        group_m = instances.BEST_GROUP_M.get(key, 8)
+    def add_gemm(name, M, K, N, f16, batch=1, gen=None):
+        inst = tuned.load(name)
 
         def build():
             if gen is not None:
@@ -42,77 +51,102 @@ def make_workloads(torch, workloads, instances):
                 A, Bm = workloads.gemm_u8s8_inputs(M, K, N, seed=2)
             shape = (batch, M, N) if batch > 1 else (M, N)
             C = torch.empty(shape, dtype=torch.float16 if f16 else torch.int32, device="cuda")
-            return dev(A), dev(Bm), C, B.gemm_problem(batch, M, N, K, group_m)
+            return dev(A), dev(Bm), C, B.gemm_problem(batch, M, N, K, inst.group_m, inst.split_k)
         ops, byts = workloads.gemm_work(M, N, K, 2 if f16 else 1, 2 if f16 else 4, batch)
-        W[name] = dict(desc=instances.BEST[key], build=build, ops=ops, bytes=byts, f16=f16,
-                       desc_text="%s batch=%d M=%d N=%d K=%d" % ("gemm_f16" if f16 else "gemm_u8s8", batch, M, N, K))
+        W[name] = dict(inst=inst, build=build, ops=ops, bytes=byts, f16=f16,
+                       text="%s batch=%d M=%d N=%d K=%d" % ("gemm_f16" if f16 else "gemm_u8s8", batch, M, N, K))
 
-    add_gemm("gemm_f16_4096", "gemm_f16_4096", 4096, 4096, 4096, True)
-    add_gemm("gemm_f16_8192", "gemm_f16", 8192, 8192, 8192, True)
-    add_gemm("gemm_u8s8_8192", "gemm_u8s8", 8192, 8192, 8192, False)
-    add_gemm("bmm_f16_qk", "bmm_f16_qk", 512, 64, 512, True, 192, lambda: workloads.bmm_qk_inputs(192, 512, 64, 512))
-    add_gemm("bmm_f16_pv", "bmm_f16_pv", 512, 512, 64, True, 192, lambda: workloads.bmm_pv_inputs(192, 512, 512, 64))
+    add_gemm("gemm_u8s8_8192", 8192, 8192, 8192, False)
+    add_gemm("gemm_f16_8192", 8192, 8192, 8192, True)
+    add_gemm("gemm_f16_4096", 4096, 4096, 4096, True)
+    add_gemm("bmm_f16_qk", 512, 64, 512, True, 192, lambda: workloads.bmm_qk_inputs(192, 512, 64, 512))
+    add_gemm("bmm_f16_pv", 512, 512, 64, True, 192, lambda: workloads.bmm_pv_inputs(192, 512, 512, 64))
 
-    def build_conv():
-        X, Wt = workloads.conv2d_inputs(32, 56, 56, 64, 64, 3, 3, seed=3)
-        Y = torch.empty((32, 56, 56, 64), dtype=torch.float16, device="cuda")
-        return dev(X), dev(Wt), Y, B.conv2d_problem(32, 56, 56, 64, 64, 3, 3, 1, 1, 1,
-                                                    instances.BEST_GROUP_M.get("conv2d_f16", 8))
-    ops, byts = workloads.conv_work(32, 56, 56, 64, 64, 3, 3, 1, 1, 1)
-    W["conv2d_f16_resnet"] = dict(desc=instances.BEST["conv2d_f16"], build=build_conv, ops=ops, bytes=byts, f16=True,
-                                  desc_text="conv2d_nhwc_f16 N=32 H=W=56 C=64 K=64 3x3 s1 p1")
+    def add_conv(name, f16):
+        inst = tuned.load(name)
 
-    def build_conv_i8():
-        X, Wt = workloads.conv2d_u8s8_inputs(32, 56, 56, 64, 64, 3, 3, seed=6)
-        Y = torch.empty((32, 56, 56, 64), dtype=torch.int32, device="cuda")
-        return dev(X), dev(Wt), Y, B.conv2d_problem(32, 56, 56, 64, 64, 3, 3, 1, 1, 1,
-                                                    instances.BEST_GROUP_M.get("conv2d_u8s8", 8))
-    ops, byts = workloads.conv_work(32, 56, 56, 64, 64, 3, 3, 1, 1, 1, in_bytes=1, out_bytes=4)
-    W["conv2d_u8s8_resnet"] = dict(desc=instances.BEST["conv2d_u8s8"], build=build_conv_i8, ops=ops, bytes=byts, f16=False,
-                                   desc_text="conv2d_nhwc_u8s8 N=32 H=W=56 C=64 K=64 3x3 s1 p1")
+        def build():
+            gen = workloads.conv2d_inputs if f16 else workloads.conv2d_u8s8_inputs
+            X, Wt = gen(32, 56, 56, 64, 64, 3, 3, seed=3 if f16 else 6)
+            Y = torch.empty((32, 56, 56, 64), dtype=torch.float16 if f16 else torch.int32, device="cuda")
+            return dev(X), dev(Wt), Y, B.conv2d_problem(32, 56, 56, 64, 64, 3, 3, 1, 1, 1, inst.group_m, inst.split_k)
+        ops, byts = workloads.conv_work(32, 56, 56, 64, 64, 3, 3, 1, 1, 1, in_bytes=2 if f16 else 1, out_bytes=2 if f16 else 4)
+        W[name] = dict(inst=inst, build=build, ops=ops, bytes=byts, f16=f16,
+                       text="conv2d_nhwc_%s N=32 H=W=56 C=64 K=64 3x3 s1 p1" % ("f16" if f16 else "u8s8"))
+
+    add_conv("conv2d_f16_resnet", True)
+    add_conv("conv2d_u8s8_resnet", False)
     return W
 
 
-def measure(torch, B, w, steps, warmup, keep_rows=0):
-    """Returns (wall seconds per step, event seconds per launch, kernel resources[, first rows of the timed output])."""
-    mod = B.Module(w["desc"])
+def settle(torch, mod, prob, a, b, c, stream, min_ms=200.0, max_ms=4000.0):
+    """Untimed clock / power warm-up with the kernel that is about to be timed: at least ``min_ms`` of launches, then
+    20-launch groups until two consecutive ones agree within 2 %.  Returns (milliseconds spent, last group's ms per
+    launch)."""
+    t0 = time.perf_counter()
+    prev, spent = None, 0.0
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    while True:
+        e0.record()
+        mod.launch_repeat(prob, a, b, c, 20, stream)
+        e1.record()
+        e1.synchronize()
+        cur = e0.elapsed_time(e1) / 20.0
+        spent = (time.perf_counter() - t0) * 1e3
+        if spent >= min_ms and prev is not None and abs(cur - prev) <= 0.02 * prev:
+            return spent, cur
+        if spent >= max_ms:
+            return spent, cur
+        prev = cur
+
+
+def measure(torch, B, w, steps, warmup, keep_rows=0, cold=False):
+    """One workload: returns dict(wall_s, kernel_s, settle_ms, info[, cold_s][, rows])."""
+    inst = w["inst"]
+    mod = B.Module(inst.desc)
     a, b, c, prob = w["build"]()
+    mod.bind_workspace(prob)
     stream = torch.cuda.current_stream().cuda_stream
+    pa, pb, pc = a.data_ptr(), b.data_ptr(), c.data_ptr()
+    spent, _ = settle(torch, mod, prob, pa, pb, pc, stream)
     if warmup > 0:
-        mod.launch_repeat(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), warmup, stream)
+        mod.launch_repeat(prob, pa, pb, pc, warmup, stream)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    mod.launch_repeat(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), steps, stream)     # exactly `steps` launches
+    e0.record()                                   # events on the launch stream (torch's current stream)
+    mod.launch_repeat(prob, pa, pb, pc, steps, stream)     # exactly `steps` launches
+    e1.record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
-    # per-launch kernel duration from HIP events recorded on the launch stream
-    costs = mod.time(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), number=steps, repeat=3, min_repeat_ms=0.0, stream=stream)
-    ev = sorted(costs)[len(costs) // 2]
-    info = dict(mod.info)
+    out = {"wall_s": wall, "kernel_s": e0.elapsed_time(e1) * 1e-3 / steps, "settle_ms": spent, "info": dict(mod.info)}
+    if cold:
+        flush = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        costs = mod.time_cold(prob, pa, pb, pc, flush.data_ptr(), flush.numel(), repeat=9, stream=stream)
+        out["cold_s"] = sorted(costs)[len(costs) // 2]
+        del flush
+    if keep_rows:
+        out["rows"] = c.reshape(-1, c.shape[-1])[:keep_rows].cpu().numpy()
     mod.close()
-    rows = c.reshape(-1, c.shape[-1])[:keep_rows].cpu().numpy() if keep_rows else None
     del a, b, c
-    return (wall, ev, info, rows) if keep_rows else (wall, ev, info)
+    return out
 
 
-# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
-# what the same counters read for the plain copy kernel of known size (profiles/ holds the runs these come from)
-MEASURED_TRAFFIC = {
-    "gemm_f16_4096": 235.0e6,     # profiles/hrn_mfma_kernel_gemm_f16_4096.md
-    "gemm_f16_8192": 1746.1e6,    # profiles/hrn_mfma_kernel_gemm_f16_8192.md
-    "gemm_u8s8_8192": 1074.4e6,   # profiles/hrn_mfma_kernel_gemm_u8s8_8192.md
-    "bmm_f16_qk": 126.0e6,        # profiles/hrn_mfma_kernel_conv_bmm.md
-    "conv2d_f16_resnet": 26.5e6,  # profiles/hrn_mfma_kernel_conv_bmm.md
-    "bmm_f16_pv": 125.9e6,        # profiles/hrn_mfma_kernel_conv_bmm.md
-    "conv2d_u8s8_resnet": 32.6e6, # profiles/hrn_mfma_kernel_conv_bmm.md
-}
-
-
-def safe_probes(torch, B):
+def traffic_table():
+    """instance -> measured HBM bytes per launch, from the tracked rocprofv3 counter runs (profiles/traffic.json)."""
     try:
-        return run_probes(torch, B)
-    except Exception as e:  # noqa: BLE001 - context figures only
-        return {"error": repr(e)[:200]}
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
+
+
+def measured_traffic(table, name, inst):
+    """Bytes per launch when the profiled instance is the one that runs now, else None."""
+    row = table.get(name)
+    if not row or row.get("instance") != list(inst.desc.as_tuple()):
+        return None
+    return row.get("bytes")
 
 
 def run_probes(torch, B):
@@ -122,42 +156,34 @@ def run_probes(torch, B):
     dst = torch.empty(n, dtype=torch.uint8, device="cuda")
     st = torch.cuda.current_stream().cuda_stream
     out = {
-        "mfma_f16_const_operands_TFLOPs": B.probe_mfma(B.HRN_DT_F16, 32, False, st),
-        "mfma_f16_random_operands_TFLOPs": B.probe_mfma(B.HRN_DT_F16, 32, True, st),
-        "mfma_i8_const_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 32, False, st),
-        "mfma_i8_random_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 32, True, st),
+        "mfma_f16_const_operands_TFLOPs": B.probe_mfma(B.HRN_DT_F16, 16, False, st),
+        "mfma_f16_random_operands_TFLOPs": B.probe_mfma(B.HRN_DT_F16, 16, True, st),
+        "mfma_i8_const_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 16, False, st),
+        "mfma_i8_random_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 16, True, st),
         "hbm_copy_1GiB_read_plus_write_GBs": B.probe_copy(src.data_ptr(), dst.data_ptr(), n, 10, st),
     }
     del src, dst
-    # the vendor library on the same random operands, for orientation only (torch.matmul = hipBLASLt / rocBLAS);
-    # a library problem must not cost the benchmark line
-    try:
-        for n in (4096, 8192):
-            a = (torch.randn(n, n, device="cuda") * 0.1).half()
-            b = (torch.randn(n, n, device="cuda") * 0.1).half()
-            for _ in range(5):
-                torch.matmul(a, b.t())
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            reps = 200 if n == 4096 else 50
-            e0.record()
-            for _ in range(reps):
-                torch.matmul(a, b.t())
-            e1.record()
-            torch.cuda.synchronize()
-            out["vendor_library_gemm_f16_%d_TFLOPs" % n] = 2.0 * n ** 3 / (e0.elapsed_time(e1) * 1e-3 / reps) / 1e12
-            del a, b
-    except Exception as e:  # noqa: BLE001
-        out["vendor_library_error"] = repr(e)[:200]
-    # the library's int8 product (signed x signed -> int32, the closest it offers to the u8 x s8 GEMM) on random bytes
+    # the vendor library on the same random operands, for orientation only; a library problem must not cost the line
     try:
         n = 8192
-        a = torch.randint(-128, 128, (n, n), device="cuda", dtype=torch.int8)
-        b = torch.randint(-128, 128, (n, n), device="cuda", dtype=torch.int8)
-        for _ in range(5):
-            torch._int_mm(a, b.t())
+        a = (torch.randn(n, n, device="cuda") * 0.1).half()
+        b = (torch.randn(n, n, device="cuda") * 0.1).half()
+        for _ in range(20):
+            torch.matmul(a, b.t())
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(50):
+            torch.matmul(a, b.t())
+        e1.record()
+        torch.cuda.synchronize()
+        out["vendor_library_gemm_f16_8192_TFLOPs"] = 2.0 * n ** 3 / (e0.elapsed_time(e1) * 1e-3 / 50) / 1e12
+        del a, b
+        a = torch.randint(-128, 128, (n, n), device="cuda", dtype=torch.int8)
+        b = torch.randint(-128, 128, (n, n), device="cuda", dtype=torch.int8)
+        for _ in range(20):
+            torch._int_mm(a, b.t())
+        torch.cuda.synchronize()
         e0.record()
         for _ in range(50):
             torch._int_mm(a, b.t())
@@ -166,105 +192,72 @@ def run_probes(torch, B):
         out["vendor_library_gemm_s8s8_8192_TOPs"] = 2.0 * n ** 3 / (e0.elapsed_time(e1) * 1e-3 / 50) / 1e12
         del a, b
     except Exception as e:  # noqa: BLE001
-        out["vendor_library_int8_error"] = repr(e)[:200]
-    # the library's convolution (torch conv2d = MIOpen) on the ResNet-50 stage-2 shape, channels-last fp16 in and out
-    try:
-        x = torch.relu(torch.randn(32, 64, 56, 56, device="cuda")).half().contiguous(memory_format=torch.channels_last)
-        w = (torch.randn(64, 64, 3, 3, device="cuda") * 0.05).half().contiguous(memory_format=torch.channels_last)
-        for _ in range(20):            # the library's first calls of a shape run a slow fallback kernel
-            torch.nn.functional.conv2d(x, w, padding=1)
-        torch.cuda.synchronize()
-        groups = []
-        for _ in range(5):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(100):
-                torch.nn.functional.conv2d(x, w, padding=1)
-            e1.record()
-            torch.cuda.synchronize()
-            groups.append(e0.elapsed_time(e1) * 1e3 / 100)
-        out["vendor_library_conv2d_f16_resnet_us"] = min(groups)
-        del x, w
-    except Exception as e:  # noqa: BLE001
-        out["vendor_library_conv_error"] = repr(e)[:200]
+        out["vendor_library_error"] = repr(e)[:200]
     return out
 
 
-def roofline(w, ev_seconds, workloads):
+def roofline(w, seconds, workloads):
+    """Roofline entry from the algorithmic work / bytes of one launch and its duration."""
     ai = w["ops"] / w["bytes"]
     peak_mfma = workloads.PEAK_FP16_TFLOPS if w["f16"] else workloads.PEAK_INT8_TOPS
     ridge = peak_mfma * 1e12 / (workloads.PEAK_HBM_GBS * 1e9)
     if ai >= ridge:
-        ach = w["ops"] / ev_seconds / 1e12
+        ach = w["ops"] / seconds / 1e12
         return {"bound": "mfma", "achieved": ach, "peak": peak_mfma, "unit": "TFLOP/s" if w["f16"] else "TOP/s",
                 "frac": ach / peak_mfma, "traffic": None}
-    ach = w["bytes"] / ev_seconds / 1e9
+    ach = w["bytes"] / seconds / 1e9
     return {"bound": "hbm", "achieved": ach, "peak": workloads.PEAK_HBM_GBS, "unit": "GB/s",
             "frac": ach / workloads.PEAK_HBM_GBS, "traffic": None}
 
 
-def cpu_baseline(name, workloads, gpu_rows=None):
-    """The CPU oracle on a bounded sample of the workload (checker code used as a reported baseline only).  When the
-    first rows of the GPU output of the timed buffers are passed in, the same sample also checks them."""
+def is_hbm_bound(w, workloads):
+    peak_mfma = workloads.PEAK_FP16_TFLOPS if w["f16"] else workloads.PEAK_INT8_TOPS
+    return w["ops"] / w["bytes"] < peak_mfma * 1e12 / (workloads.PEAK_HBM_GBS * 1e9)
+
+
+def cpu_baseline(workloads, gpu_rows=None):
+    """The CPU oracle's DL Boost-style GEMM on the 8192^3 problem (checker code used as a reported baseline only);
+    the first rows of the GPU output of the timed buffers are checked against the same result."""
     import numpy as np
     import oracle
     cores = len(os.sched_getaffinity(0))
-    if name.startswith("gemm_u8s8"):
-        M, K, N = 8192, 8192, 8192
-        A, Bm = workloads.gemm_u8s8_inputs(M, K, N, seed=2)
-        if oracle.has_vnni():
-            pb = oracle.PackedB(Bm)
-            C = np.empty((M, N), np.int32)
-            pb.matmul(A[:256], out=C[:256])                # warm-up
-            reps, t0 = 0, time.perf_counter()
-            while True:
-                pb.matmul(A, out=C)
-                reps += 1
-                if time.perf_counter() - t0 > 10 or reps >= 20:
-                    break
-            dt = (time.perf_counter() - t0) / reps
-            out = {"value": 2.0 * M * N * K / dt / 1e12, "unit": "TOP/s", "cores": oracle.num_threads(), "kind": "port",
-                   "sample": "full 8192^3 u8s8 GEMM x%d, AVX512-VNNI 16x4 vpdpbusd micro-kernel, B pre-packed, "
-                             "%d OpenMP threads of %d host cores" % (reps, oracle.num_threads(), cores)}
-            if gpu_rows is not None:
-                out["gpu_rows_bit_exact"] = bool(np.array_equal(gpu_rows, C[:len(gpu_rows)]))
-            return out
-        rows = 64
-        t0 = time.perf_counter()
-        oracle.gemm_u8s8s32_dlboost(A[:rows], Bm)
-        dt = time.perf_counter() - t0
-        return {"value": 2.0 * rows * N * K / dt / 1e12, "unit": "TOP/s", "cores": oracle.num_threads(), "kind": "port",
-                "sample": "%d rows of the 8192^3 u8s8 GEMM, scalar fallback (no AVX512-VNNI)" % rows}
-    # fp16 workloads: fp32 host reference (double accumulate) on a slab of rows
-    M, K, N = 4096, 4096, 4096
-    A, Bm = workloads.gemm_f16_inputs(M, K, N, seed=1)
+    M = K = N = 8192
+    A, Bm = workloads.gemm_u8s8_inputs(M, K, N, seed=2)
+    if oracle.has_vnni():
+        pb = oracle.PackedB(Bm)
+        C = np.empty((M, N), np.int32)
+        pb.matmul(A[:256], out=C[:256])                # warm-up
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            pb.matmul(A, out=C)
+            reps += 1
+            if time.perf_counter() - t0 > 10 or reps >= 20:
+                break
+        dt = (time.perf_counter() - t0) / reps
+        out = {"value": 2.0 * M * N * K / dt / 1e12, "unit": "TOP/s", "cores": oracle.num_threads(), "kind": "port",
+               "sample": "full 8192^3 u8s8 GEMM x%d, AVX512-VNNI 16x4 vpdpbusd micro-kernel, B pre-packed, "
+                         "%d OpenMP threads of %d host cores" % (reps, oracle.num_threads(), cores)}
+        if gpu_rows is not None:
+            out["gpu_rows_bit_exact"] = bool(np.array_equal(gpu_rows, C[:len(gpu_rows)]))
+        return out
     rows = 64
-    Af, Bf = A[:rows].astype(np.float32), Bm.astype(np.float32)
-    oracle.gemm_f32(Af[:8], Bf)
     t0 = time.perf_counter()
-    reps = 0
-    while True:
-        oracle.gemm_f32(Af, Bf)
-        reps += 1
-        if time.perf_counter() - t0 > 10 or reps >= 50:
-            break
-    dt = (time.perf_counter() - t0) / reps
-    out = {"value": 2.0 * rows * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
-           "sample": "%d of 4096 rows of the fp16 GEMM 4096^3 x%d, fp32 host reference (double accumulate), "
-                     "%d OpenMP threads of %d host cores" % (rows, reps, oracle.num_threads(), cores)}
+    ref = oracle.gemm_u8s8s32_dlboost(A[:rows], Bm)
+    dt = time.perf_counter() - t0
+    out = {"value": 2.0 * rows * N * K / dt / 1e12, "unit": "TOP/s", "cores": oracle.num_threads(), "kind": "port",
+           "sample": "%d rows of the 8192^3 u8s8 GEMM, scalar fallback (no AVX512-VNNI)" % rows}
     if gpu_rows is not None:
-        ref = oracle.gemm_f32(Af[:len(gpu_rows)], Bf)
-        out["gpu_rows_max_rel_err"] = float(np.abs(gpu_rows.astype(np.float32) - ref).max() / np.abs(ref).max())
+        out["gpu_rows_bit_exact"] = bool(np.array_equal(gpu_rows[:rows], ref[:len(gpu_rows)]))
     return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=1000)
-    ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="gemm_f16_4096")
-    ap.add_argument("--only", action="store_true", help="skip the 'also' workloads and the CPU baseline")
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default=HEADLINE)
+    ap.add_argument("--only", action="store_true", help="skip the 'also' workloads, the probes and the CPU baseline")
     ap.add_argument("--probe", action="store_true", help="only run the roofline probes (MFMA loop, 1 GiB copy)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -274,7 +267,7 @@ def main():
 
     import torch
     from heron_amd import backend as B
-    from heron_amd import instances, workloads
+    from heron_amd import tuned, workloads
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
@@ -282,58 +275,68 @@ def main():
     if args.probe:
         print(json.dumps({"probes": run_probes(torch, B)}))
         return
-    W = make_workloads(torch, workloads, instances)
-    if args.workload not in W:
-        print("unknown workload %s (have %s)" % (args.workload, sorted(W)), file=sys.stderr)
+    if args.workload not in tuned.CASES:
+        print("unknown workload %s (have %s)" % (args.workload, sorted(tuned.CASES)), file=sys.stderr)
         sys.exit(2)
+    W = make_workloads(torch, workloads, tuned)
+    table = traffic_table()
 
     w = W[args.workload]
-    check_rows = 64 if (args.workload in ("gemm_f16_4096", "gemm_u8s8_8192") and not args.only) else 0
-    if check_rows:
-        wall, ev, info, gpu_rows = measure(torch, B, w, args.steps, args.warmup, check_rows)
-    else:
-        (wall, ev, info), gpu_rows = measure(torch, B, w, args.steps, args.warmup), None
+    inst = w["inst"]
+    check = args.workload == HEADLINE and not args.only
+    r = measure(torch, B, w, args.steps, args.warmup, keep_rows=64 if check else 0, cold=is_hbm_bound(w, workloads))
+    roof = roofline(w, r.get("cold_s", r["kernel_s"]), workloads)
+    roof["traffic"] = measured_traffic(table, args.workload, inst)
     line = {
         "metric": "%s throughput per GPU (tuned MFMA template)" % ("fp16 GEMM TFLOPS" if w["f16"] else "u8s8 GEMM TOPS"),
-        "value": w["ops"] / wall / 1e12,
+        "value": w["ops"] / r["wall_s"] / 1e12,
         "unit": "TFLOP/s" if w["f16"] else "TOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": wall * 1e3,
+        "ms_per_step": r["wall_s"] * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16" if w["f16"] else "u8",
         "data": "synthetic",
-        "config": {"workload": w["desc_text"], "instance": repr(w["desc"]), "kernel_ms": ev * 1e3, "resources": info},
-        "roofline": roofline(w, ev, workloads),
+        "config": {"workload": w["text"], "instance": repr(inst.desc), "record": inst.code,
+                   "records_file": os.path.relpath(inst.records, ROOT), "group_m": inst.group_m, "split_k": inst.split_k,
+                   "kernel_ms": r["kernel_s"] * 1e3, "clock_settle_ms": r["settle_ms"], "resources": r["info"]},
+        "roofline": roof,
     }
-    line["roofline"]["traffic"] = MEASURED_TRAFFIC.get(args.workload)
-    line["peaks"] = {"published": {"mfma_f16_TFLOPs": workloads.PEAK_FP16_TFLOPS, "mfma_i8_TOPs": workloads.PEAK_INT8_TOPS,
-                                   "hbm_GBs": workloads.PEAK_HBM_GBS},
-                     "measured": safe_probes(torch, B), "used": "published"}
+    if "cold_s" in r:
+        line["config"]["kernel_ms_cold"] = r["cold_s"] * 1e3
     if not args.only:
+        line["peaks"] = {"published": {"mfma_f16_TFLOPs": workloads.PEAK_FP16_TFLOPS, "mfma_i8_TOPs": workloads.PEAK_INT8_TOPS,
+                                       "hbm_GBs": workloads.PEAK_HBM_GBS}, "used": "published"}
+        try:
+            line["peaks"]["measured"] = run_probes(torch, B)
+        except Exception as e:  # noqa: BLE001 - context figures only
+            line["peaks"]["measured"] = {"error": repr(e)[:200]}
         also = []
         for name, ww in W.items():
             if name == args.workload:
                 continue
-            steps = max(10, min(args.steps, 500))
+            steps = max(10, min(args.steps, 200))
+            hbm = is_hbm_bound(ww, workloads)
             try:
-                wl, e, _ = measure(torch, B, ww, steps, min(args.warmup, 5))
+                rr = measure(torch, B, ww, steps, min(args.warmup, 5), cold=hbm)
             except Exception as err:  # noqa: BLE001 - one side workload must not cost the headline
-                also.append({"workload": ww["desc_text"], "error": repr(err)[:200]})
+                also.append({"workload": ww["text"], "error": repr(err)[:200]})
                 continue
-            r = roofline(ww, e, workloads)
-            r["traffic"] = MEASURED_TRAFFIC.get(name)
-            also.append({"workload": ww["desc_text"], "value": ww["ops"] / wl / 1e12,
-                         "unit": "TFLOP/s" if ww["f16"] else "TOP/s", "steps": steps, "kernel_ms": e * 1e3,
-                         "frac_of_mfma_peak": ww["ops"] / e / 1e12 / (workloads.PEAK_FP16_TFLOPS if ww["f16"] else workloads.PEAK_INT8_TOPS),
-                         "roofline": r})
+            rf = roofline(ww, rr.get("cold_s", rr["kernel_s"]), workloads)
+            rf["traffic"] = measured_traffic(table, name, ww["inst"])
+            peak = workloads.PEAK_FP16_TFLOPS if ww["f16"] else workloads.PEAK_INT8_TOPS
+            row = {"workload": ww["text"], "value": ww["ops"] / rr["wall_s"] / 1e12,
+                   "unit": "TFLOP/s" if ww["f16"] else "TOP/s", "steps": steps, "kernel_ms": rr["kernel_s"] * 1e3,
+                   "record": ww["inst"].code, "instance": list(ww["inst"].desc.as_tuple()),
+                   "frac_of_mfma_peak": ww["ops"] / rr["kernel_s"] / 1e12 / peak, "roofline": rf}
+            if "cold_s" in rr:
+                row["kernel_ms_cold"] = rr["cold_s"] * 1e3
+                row["roofline_timed"] = "cold: every launch after 1 GiB was streamed through the caches"
+            also.append(row)
         line["also"] = also
-        def guarded(*a):
-            try:
-                return cpu_baseline(*a)
-            except Exception as e:  # noqa: BLE001 - the GPU figures above are still worth printing
-                return {"value": None, "unit": None, "cores": 0, "kind": "port", "sample": "failed: %r" % (e,)}
-        line["cpu_baseline"] = guarded(args.workload, workloads, gpu_rows)
-        line["cpu_baseline_u8s8"] = guarded("gemm_u8s8_8192", workloads) if not args.workload.startswith("gemm_u8s8") else None
+        try:
+            line["cpu_baseline"] = cpu_baseline(workloads, r.get("rows") if args.workload == HEADLINE else None)
+        except Exception as e:  # noqa: BLE001 - the GPU figures above are still worth printing
+            line["cpu_baseline"] = {"value": None, "unit": None, "cores": 0, "kind": "port", "sample": "failed: %r" % (e,)}
     print(json.dumps(line))
 
 

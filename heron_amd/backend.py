@@ -49,11 +49,12 @@ class KernelDesc(ctypes.Structure):
     _fields_ = [("dtype", ctypes.c_int32), ("op", ctypes.c_int32), ("bm", ctypes.c_int32), ("bn", ctypes.c_int32),
                 ("bkb", ctypes.c_int32), ("wm", ctypes.c_int32), ("wn", ctypes.c_int32), ("mfma", ctypes.c_int32),
                 ("stages", ctypes.c_int32), ("swizzle", ctypes.c_int32), ("epilogue", ctypes.c_int32),
-                ("waves_per_eu", ctypes.c_int32), ("l2_prefetch", ctypes.c_int32), ("ablate", ctypes.c_int32),
-                ("load_mode", ctypes.c_int32), ("conv_window", ctypes.c_int32), ("persistent", ctypes.c_int32)]
+                ("waves_per_eu", ctypes.c_int32), ("conv_window", ctypes.c_int32), ("persistent", ctypes.c_int32),
+                ("split_k", ctypes.c_int32), ("sched", ctypes.c_int32),
+                ("load_spread", ctypes.c_int32)]
 
     KEYS = ("dtype", "op", "bm", "bn", "bkb", "wm", "wn", "mfma", "stages", "swizzle", "epilogue", "waves_per_eu",
-            "l2_prefetch", "ablate", "load_mode", "conv_window", "persistent")
+            "conv_window", "persistent", "split_k", "sched", "load_spread")
 
     def as_tuple(self):
         return tuple(int(getattr(self, k)) for k in self.KEYS)
@@ -80,14 +81,14 @@ class Problem(ctypes.Structure):
                 ("co", ctypes.c_int32), ("kh", ctypes.c_int32), ("kw", ctypes.c_int32),
                 ("cstride", ctypes.c_int32), ("cpad", ctypes.c_int32), ("cdil", ctypes.c_int32),
                 ("group_m", ctypes.c_int32),
-                ("cstride_w", ctypes.c_int32), ("cpad_w", ctypes.c_int32), ("cdil_w", ctypes.c_int32)]
+                ("cstride_w", ctypes.c_int32), ("cpad_w", ctypes.c_int32), ("cdil_w", ctypes.c_int32),
+                ("split_k", ctypes.c_int32), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t)]
 
 
 def make_desc(dtype, op=HRN_OP_GEMM, bm=128, bn=128, bkb=128, wm=2, wn=2, mfma=32, stages=2, swizzle=1,
-              epilogue=0, waves_per_eu=0, l2_prefetch=0, ablate=0, load_mode=0, conv_window=0, persistent=0):
+              epilogue=0, waves_per_eu=0, conv_window=0, persistent=0, split_k=0, sched=1, load_spread=2):
     d = KernelDesc()
-    d.l2_prefetch, d.ablate, d.load_mode, d.conv_window = l2_prefetch, ablate, load_mode, conv_window
-    d.persistent = persistent
+    d.conv_window, d.persistent, d.split_k, d.sched, d.load_spread = conv_window, persistent, split_k, sched, load_spread
     d.dtype, d.op, d.bm, d.bn, d.bkb, d.wm, d.wn = dtype, op, bm, bn, bkb, wm, wn
     d.mfma, d.stages, d.swizzle, d.epilogue, d.waves_per_eu = mfma, stages, swizzle, epilogue, waves_per_eu
     return d
@@ -133,6 +134,7 @@ SYMBOLS = {
     "hrn_launch_repeat": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _vp]),
     "hrn_time": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _i, _d, ctypes.POINTER(_d), _vp]),
     "hrn_time_cold": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
+    "hrn_splitk_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(KernelDesc), ctypes.POINTER(Problem)]),
     "hrn_problem_gemm": (None, [ctypes.POINTER(Problem), _i, _i, _i, _i]),
     "hrn_problem_conv2d": (None, [ctypes.POINTER(Problem)] + [_i] * 10),
     "hrn_problem_conv2d_hw": (None, [ctypes.POINTER(Problem)] + [_i] * 13),
@@ -190,23 +192,33 @@ def compile_desc(desc, timeout_s=0.0):
     return buf.value.decode()
 
 
-def gemm_problem(batch, m, n, k, group_m=8):
+def gemm_problem(batch, m, n, k, group_m=8, split_k=0):
     p = Problem()
     lib().hrn_problem_gemm(ctypes.byref(p), batch, m, n, k)
     p.group_m = group_m
+    p.split_k = split_k
     return p
+
+
+def splitk_workspace_bytes(desc, problem):
+    """Bytes of device workspace a split-K launch of ``desc`` on ``problem`` needs (0 for other instances)."""
+    n = lib().hrn_splitk_workspace_bytes(ctypes.byref(desc), ctypes.byref(problem))
+    if n < 0:
+        _check(int(n))
+    return int(n)
 
 
 def _pair(v):
     return (int(v), int(v)) if isinstance(v, int) else (int(v[0]), int(v[1]))
 
 
-def conv2d_problem(n, h, w, ci, co, kh, kw, stride, pad, dil, group_m=8):
+def conv2d_problem(n, h, w, ci, co, kh, kw, stride, pad, dil, group_m=8, split_k=0):
     """``stride``, ``pad`` and ``dil`` are ints or (height, width) pairs."""
     p = Problem()
     (sh, sw), (ph, pw), (dh, dw) = _pair(stride), _pair(pad), _pair(dil)
     lib().hrn_problem_conv2d_hw(ctypes.byref(p), n, h, w, ci, co, kh, kw, sh, sw, ph, pw, dh, dw)
     p.group_m = group_m
+    p.split_k = split_k
     return p
 
 
@@ -236,6 +248,22 @@ class Module:
         _check(lib().hrn_module_info(self._h, ctypes.byref(info)))
         self.info = info.as_dict()
 
+    def bind_workspace(self, problem):
+        """Split-K instances: point ``problem`` at a device workspace owned by this module (torch supplies the
+        memory; it grows on demand and is shared by the launches of this module, which therefore must not overlap)."""
+        if not self.desc.split_k or problem.workspace:
+            return problem
+        if problem.split_k < 1:
+            problem.split_k = 1
+        need = splitk_workspace_bytes(self.desc, problem)
+        ws = getattr(self, "_ws", None)
+        if ws is None or ws.numel() < need:
+            import torch
+            self._ws = ws = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device="cuda")
+        problem.workspace = ws.data_ptr()
+        problem.workspace_bytes = ws.numel()
+        return problem
+
     def _launcher(self, problem):
         L = lib()
         if self.desc.op == HRN_OP_CONV2D:
@@ -245,20 +273,24 @@ class Module:
         return L.hrn_launch_bmm_f16 if problem.batch > 1 else L.hrn_launch_gemm_f16
 
     def launch(self, problem, a_ptr, b_ptr, c_ptr, stream=0):
+        self.bind_workspace(problem)
         _check(self._launcher(problem)(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, stream))
 
     def launch_repeat(self, problem, a_ptr, b_ptr, c_ptr, count, stream=0):
         """``count`` back-to-back launches issued from one host call."""
+        self.bind_workspace(problem)
         _check(lib().hrn_launch_repeat(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, count, stream))
 
     def time_cold(self, problem, a_ptr, b_ptr, c_ptr, flush_ptr, flush_bytes, repeat=4, stream=0):
         """Seconds of ``repeat`` single launches, each after the caches were flushed with the caller's buffer."""
+        self.bind_workspace(problem)
         costs = (_d * repeat)()
         _check(lib().hrn_time_cold(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, flush_ptr, flush_bytes, repeat,
                                    costs, stream))
         return list(costs)
 
     def time(self, problem, a_ptr, b_ptr, c_ptr, number=3, repeat=4, min_repeat_ms=0.0, stream=0):
+        self.bind_workspace(problem)
         costs = (_d * repeat)()
         _check(lib().hrn_time(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, number, repeat,
                               float(min_repeat_ms), costs, stream))
@@ -268,6 +300,7 @@ class Module:
         if getattr(self, "_h", None):
             lib().hrn_module_free(self._h)
             self._h = None
+        self._ws = None
 
     def __del__(self):
         try:

@@ -1,55 +1,46 @@
-"""Tuning configuration: defaults and JSON schema of the reference (config.py:4-54)."""
+"""Tuning configuration.  Field names, defaults and the JSON schema of a case file are the reference's
+(config.py:4-54): ``{"config": {"out_name", "method", "max_trials", "runner_number", "runner_repeat",
+"runner_timeout", "build_timeout", "in_dtype", "out_dtype", "cases": {name: [op, shape]}, ["temperature"]}}``."""
 import json
 import os
+
+# attribute -> default; grouped as the reference groups them
+DEFAULTS = {
+    # environment
+    'target_name': None, 'codegen_type': None, 'get_op': None, 'verbose': False, 'measure_time_per_round': 32,
+    'use_cost_model': True, 'out_name': 'out', 'device_id': 0, 'tuned': '',
+    # sampling processes
+    'parallel': True, 'parallel_num': 16,
+    # population
+    'pop_num': 200, 'iter_walks': 5, 'history_topk': 32,
+    # cost model
+    'feature_type': 'itervar', 'loss_type': 'reg',
+    # genetic algorithm
+    'select_num': 100, 'crossover_key_ratio': 0.2,
+    # simulated annealing
+    'temperature': 0.6,
+    # unconstrained tuners: per-variable feasible value sets from this many random feasible points (tuner.py:115-144)
+    'feasible_file_path': 'feasible.json', 'feasible_samples': 1000,
+    # cross-task cost model: rounds of run_with_pretrained (the reference reads it, tuner.py:36, but never defines it)
+    'search_generations': 4, 'pretrained_records': (),
+    # what a JSON file normally supplies
+    'opt_method': 'CGA', 'max_trials': 32, 'runner_number': 3, 'runner_repeat': 4, 'runner_timeout': 50,
+    'build_timeout': 50, 'in_dtype': 'float16', 'out_dtype': 'float16', 'cases': (),
+}
+
+# JSON key -> attribute, for the keys every case file carries
+REQUIRED_KEYS = {'out_name': 'out_name', 'method': 'opt_method', 'max_trials': 'max_trials',
+                 'runner_number': 'runner_number', 'runner_repeat': 'runner_repeat', 'runner_timeout': 'runner_timeout',
+                 'build_timeout': 'build_timeout', 'in_dtype': 'in_dtype', 'out_dtype': 'out_dtype', 'cases': 'cases'}
+# optional keys; all but "temperature" are additions of this build
+OPTIONAL_KEYS = ('temperature', 'pop_num', 'iter_walks', 'parallel_num', 'measure_time_per_round', 'select_num',
+                 'history_topk')
 
 
 class Config:
     def __init__(self):
-        # Environment configs
-        self.target_name = None
-        self.codegen_type = None
-        self.get_op = None
-        self.verbose = False
-        self.measure_time_per_round = 32
-        self.use_cost_model = True
-        self.out_name = 'out'
-        self.device_id = 0
-        self.tuned = ''
-
-        self.parallel = True
-        self.parallel_num = 16
-
-        # Common
-        self.pop_num = 200
-        self.iter_walks = 5
-        self.history_topk = 32
-
-        # cost model configs
-        self.feature_type = 'itervar'
-        self.loss_type = 'reg'
-
-        # Genetic algorithm params
-        self.select_num = 100
-        self.crossover_key_ratio = 0.2
-
-        # Simulated annealing params
-        self.temperature = 0.6
-
-        self.feasible_file_path = 'feasible.json'
-        self.search_generations = 4           # rounds of run_with_pretrained (tuner.py:36; the reference leaves it undefined)
-        self.pretrained_records = []          # records.txt files of earlier tasks for the cross-task cost model
-        self.feasible_samples = 1000          # random feasible points behind the per-variable value sets (tuner.py:115)
-
-        # defaults for configs created in code rather than from a file
-        self.opt_method = 'CGA'
-        self.max_trials = 32
-        self.runner_number = 3
-        self.runner_repeat = 4
-        self.runner_timeout = 50
-        self.build_timeout = 50
-        self.in_dtype = 'float16'
-        self.out_dtype = 'float16'
-        self.cases = {}
+        for name, value in DEFAULTS.items():
+            setattr(self, name, {} if name == 'cases' else [] if name == 'pretrained_records' else value)
 
     def setEnv(self, env):
         self.num_ops = env.num_ops
@@ -57,24 +48,12 @@ class Config:
 
 
 def configFromFile(fname):
-    with open(fname, "r") as f:
-        data = json.load(f)
+    with open(fname) as f:
+        entries = json.load(f)['config']
     config = Config()
-    c = data['config']
-    config.out_name = c['out_name']
-    config.opt_method = c['method']
-    config.max_trials = c['max_trials']
-    config.runner_number = c['runner_number']
-    config.runner_repeat = c['runner_repeat']
-    config.runner_timeout = c['runner_timeout']
-    config.build_timeout = c['build_timeout']
-    config.in_dtype = c['in_dtype']
-    config.out_dtype = c['out_dtype']
-    config.cases = c['cases']
-    if "temperature" in c.keys():
-        config.temperature = c["temperature"]
-    # optional overrides of the search defaults (not in the reference's schema)
-    for key in ("pop_num", "iter_walks", "parallel_num", "measure_time_per_round", "select_num", "history_topk"):
-        if key in c:
-            setattr(config, key, c[key])
+    for key, attr in REQUIRED_KEYS.items():
+        setattr(config, attr, entries[key])
+    for key in OPTIONAL_KEYS:
+        if key in entries:
+            setattr(config, key, entries[key])
     return config

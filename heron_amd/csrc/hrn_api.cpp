@@ -36,8 +36,8 @@ struct HrnKArgs {  // must match mfma_gemm_template.hip
     int64_t sA, sB, sC;
     int32_t tiles_m, tiles_n, group_m, batch;
     int32_t H, W, CI, HO, WO, KH, KW, cstride, cpad, cdil;
-    int32_t pf_sa, pf_sb;
     int32_t cstride_w, cpad_w, cdil_w;
+    int32_t split, kt_per_slice;
 };
 
 struct hrn_module {
@@ -47,6 +47,7 @@ struct hrn_module {
     hipFunction_t fn;
     std::string path;
     int persist_grid;   // persistent instances: workgroups that fit the device at once (multiple of 8 when >= 8)
+    int epi_bytes;      // LDS bytes of the epilogue region (column sums + strips)
 };
 
 namespace {
@@ -117,7 +118,7 @@ uint64_t fnv1a_file(const std::string& p) {
 }
 
 struct Derived {
-    int es, nw, cpr, rpi, a_lpw, b_lpw, lpt, ksb, ks, tm, tn, stage_bytes, lds;
+    int es, oes, nw, cpr, rpi, a_lpw, b_lpw, lpt, ksb, ks, tm, tn, stage_bytes, lds, epi_bytes;
 };
 
 // Structural constraints of the template; the same conditions are static_asserts in the kernel.
@@ -128,22 +129,24 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (d->bkb != 64 && d->bkb != 128 && d->bkb != 256) return fail(HRN_E_BADPARAM, "bkb %d not in {64,128,256}", d->bkb);
     if (d->mfma != 32 && d->mfma != 16) return fail(HRN_E_BADPARAM, "mfma %d not in {16,32}", d->mfma);
     if (d->wm < 1 || d->wn < 1 || d->wm * d->wn > 16) return fail(HRN_E_BADPARAM, "wave grid %dx%d", d->wm, d->wn);
+    if (d->wm & (d->wm - 1)) return fail(HRN_E_BADPARAM, "wave rows %d must be a power of two", d->wm);
     if (d->bm < 16 || d->bn < 16 || d->bm > 512 || d->bn > 512) return fail(HRN_E_BADPARAM, "tile %dx%d", d->bm, d->bn);
     if (d->stages < 2 || d->stages > 5) return fail(HRN_E_BADPARAM, "stages %d not in 2..5", d->stages);
     if (d->swizzle < 0 || d->swizzle > 3) return fail(HRN_E_BADPARAM, "swizzle %d", d->swizzle);
-    if (d->epilogue < 0 || d->epilogue > 1) return fail(HRN_E_BADPARAM, "epilogue %d", d->epilogue);
+    if (d->epilogue < 0 || d->epilogue > 2) return fail(HRN_E_BADPARAM, "epilogue %d", d->epilogue);
+    if (d->sched < 0 || d->sched > 1) return fail(HRN_E_BADPARAM, "sched %d", d->sched);
+    if (d->load_spread < 0 || d->load_spread > 3) return fail(HRN_E_BADPARAM, "load_spread %d", d->load_spread);
     if (d->waves_per_eu < 0 || d->waves_per_eu > 8) return fail(HRN_E_BADPARAM, "waves_per_eu %d", d->waves_per_eu);
-    if (d->l2_prefetch < 0 || d->l2_prefetch > 8) return fail(HRN_E_BADPARAM, "l2_prefetch %d not in 0..8", d->l2_prefetch);
-    if (d->load_mode < 0 || d->load_mode > 1) return fail(HRN_E_BADPARAM, "load_mode %d", d->load_mode);
     if (d->conv_window < 0 || d->conv_window > 1) return fail(HRN_E_BADPARAM, "conv_window %d", d->conv_window);
-    if (d->conv_window && (d->op != HRN_OP_CONV2D || d->load_mode || d->l2_prefetch))
-        return fail(HRN_E_BADPARAM, "conv_window is a conv2d option (load_mode 0, no l2_prefetch)");
-    if (d->load_mode == 1 && (d->stages != 2 || d->l2_prefetch)) return fail(HRN_E_BADPARAM, "load_mode 1 needs stages == 2 and no l2_prefetch");
+    if (d->conv_window && d->op != HRN_OP_CONV2D) return fail(HRN_E_BADPARAM, "conv_window is a conv2d option");
     if (d->persistent < 0 || d->persistent > 1) return fail(HRN_E_BADPARAM, "persistent %d", d->persistent);
-    if (d->persistent && (d->epilogue != 1 || d->load_mode || d->l2_prefetch || d->conv_window || d->ablate))
-        return fail(HRN_E_BADPARAM, "persistent needs the LDS-staged epilogue and none of load_mode, l2_prefetch, conv_window, ablate");
+    if (d->split_k < 0 || d->split_k > 1) return fail(HRN_E_BADPARAM, "split_k %d", d->split_k);
+    if (d->persistent && (d->epilogue < 1 || d->conv_window || d->split_k))
+        return fail(HRN_E_BADPARAM, "persistent needs the LDS-staged epilogue and neither conv_window nor split_k");
+    if (d->split_k && d->conv_window) return fail(HRN_E_BADPARAM, "split_k uses the im2col load path, not conv_window");
     Derived r;
     r.es = d->dtype == HRN_DT_F16 ? 2 : 1;
+    r.oes = (d->dtype == HRN_DT_F16 && !d->split_k) ? 2 : 4;
     r.nw = d->wm * d->wn;
     r.cpr = d->bkb / 16;
     r.rpi = 64 / r.cpr;
@@ -155,55 +158,53 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     r.lpt = r.a_lpw + r.b_lpw;
     r.ksb = d->mfma == 32 ? 32 : 64;
     r.ks = d->bkb / r.ksb;
-    if (r.ks < 2 || r.ks % 2) return fail(HRN_E_BADPARAM, "bkb %d gives %d k-steps for mfma %d (need even >= 2)", d->bkb, r.ks, d->mfma);
+    if (r.ks < 1) return fail(HRN_E_BADPARAM, "bkb %d is less than one k-step of mfma %d", d->bkb, d->mfma);
+    if (d->persistent && r.ks % 2) return fail(HRN_E_BADPARAM, "persistent needs an even number of k-steps per tile (bkb %d, mfma %d)", d->bkb, d->mfma);
     if (d->bm % (d->wm * d->mfma) || d->bn % (d->wn * d->mfma))
         return fail(HRN_E_BADPARAM, "tile %dx%d not divisible by wave grid %dx%d x mfma %d", d->bm, d->bn, d->wm, d->wn, d->mfma);
     r.tm = d->bm / d->wm / d->mfma;
     r.tn = d->bn / d->wn / d->mfma;
     r.stage_bytes = ((d->conv_window ? 0 : d->bm) + d->bn) * d->bkb;
-    r.lds = d->stages * r.stage_bytes + (d->l2_prefetch ? r.nw * 256 : 0);
-    if (d->epilogue == 1) {
-        const int oes = d->dtype == HRN_DT_F16 ? 2 : 4;
-        const int wtn = d->bn / d->wn;
-        const int base = d->dtype == HRN_DT_U8S8 ? ((d->bn * 4 + 1023) / 1024) * 1024 : 0;
-        const int epi = base + r.nw * d->mfma * (wtn * oes + 16);
-        if ((d->mfma * (wtn * oes / 16)) % 64) return fail(HRN_E_BADPARAM, "staged epilogue needs mfma*wave_tile_n*out_bytes/16 %% 64 == 0");
+    r.lds = d->stages * r.stage_bytes;
+    // epilogue region: the uint8 path's column sums (one row of bn sums per wave row) and, for the staged epilogue, the strips
+    const int base = d->dtype == HRN_DT_U8S8 ? ((d->wm * d->bn * 4 + 1023) / 1024) * 1024 : 0;
+    r.epi_bytes = base;
+    if (d->epilogue >= 1) {
+        const int esplit = d->epilogue == 2 ? 2 : 1;
+        if (r.tn % esplit) return fail(HRN_E_BADPARAM, "epilogue 2 needs an even number of MFMA column tiles per wave (%d)", r.tn);
+        const int sw = d->bn / d->wn / esplit;              // outputs per strip row
+        r.epi_bytes = base + r.nw * d->mfma * (sw * r.oes + 16);
+        if ((d->mfma * (sw * r.oes / 16)) % 64) return fail(HRN_E_BADPARAM, "staged epilogue needs mfma*strip_width*out_bytes/16 %% 64 == 0");
         if (d->persistent) {
             // the stages stay live during the epilogue, and its stores share the 6-bit vector-memory counter with the fetches
-            r.lds += epi;
-            const int stores = r.tm * (d->mfma * (wtn * oes / 16) / 64);
+            r.lds += r.epi_bytes;
+            const int stores = r.tm * esplit * (d->mfma * (sw * r.oes / 16) / 64);
             if ((d->stages - 2) * r.lpt + stores > 63)
                 return fail(HRN_E_BADPARAM, "persistent: %d fetches + %d stores in flight exceed 63", (d->stages - 2) * r.lpt, stores);
-        } else {
-            r.lds = std::max(r.lds, epi);
+        } else if (!d->conv_window) {
+            r.lds = std::max(r.lds, r.epi_bytes);
         }
     }
+    // (a conv_window instance keeps the epilogue region in its dynamic LDS, where the window was)
     if (r.lds > 163840) return fail(HRN_E_BADPARAM, "LDS %d > 163840", r.lds);
     if (d->swizzle && (r.cpr << (d->swizzle - 1)) > d->mfma)
         return fail(HRN_E_BADPARAM, "swizzle %d period %d exceeds mfma %d", d->swizzle, r.cpr << (d->swizzle - 1), d->mfma);
     if (d->op == HRN_OP_CONV2D && !d->conv_window && d->swizzle && (r.nw * r.rpi) % (r.cpr << (d->swizzle - 1)))
         return fail(HRN_E_BADPARAM, "conv: swizzle period must divide rows per load round");
-    {
-        // every tile fetch may be preceded by the prefetch touches of a later tile
-        if (d->l2_prefetch && d->op != HRN_OP_GEMM) return fail(HRN_E_BADPARAM, "l2_prefetch is for GEMM only");
-        if (d->l2_prefetch && r.nw < 2) return fail(HRN_E_BADPARAM, "l2_prefetch needs at least two waves");
-        const int pf = d->l2_prefetch ? 1 : 0;
-        if ((d->stages - 1) * (r.lpt + pf) > 63)
-            return fail(HRN_E_BADPARAM, "too many loads in flight (%d)", (d->stages - 1) * (r.lpt + pf));
-    }
+    if ((d->stages - 1) * r.lpt > 63) return fail(HRN_E_BADPARAM, "too many loads in flight (%d)", (d->stages - 1) * r.lpt);
     const int acc = r.tm * r.tn * (d->mfma == 32 ? 16 : 4);
     if (acc > 256) return fail(HRN_E_BADPARAM, "accumulators %d > 256 registers per lane", acc);
-    if (d->dtype == HRN_DT_U8S8 && d->bn * 4 > r.lds) return fail(HRN_E_BADPARAM, "LDS too small for the column sums");
+    if (d->dtype == HRN_DT_U8S8 && !d->conv_window && d->wm * d->bn * 4 > d->stages * r.stage_bytes)
+        return fail(HRN_E_BADPARAM, "LDS stages too small for the column sums");
     if (o) *o = r;
     return HRN_OK;
 }
 
 std::string desc_key(const hrn_kernel_desc* d, uint64_t srch) {
     char b[256];
-    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_a%d_f%d_l%d_c%d_r%d_%08x", d->dtype, d->op, d->bm, d->bn,
-             d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu, d->ablate, d->l2_prefetch, d->load_mode, d->conv_window,
-             d->persistent,
-             (unsigned)(srch ^ (srch >> 32)));
+    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_c%d_r%d_k%d_i%d_l%d_%08x", d->dtype, d->op, d->bm, d->bn,
+             d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu, d->conv_window,
+             d->persistent, d->split_k, d->sched, d->load_spread, (unsigned)(srch ^ (srch >> 32)));
     return b;
 }
 
@@ -214,18 +215,21 @@ int parse_remark(const std::string& log, const char* tag) {
 }
 
 int run_hipcc(const std::vector<std::string>& args, const std::string& log_path, double timeout_s) {
+    // everything the child needs is prepared here: between fork and exec it only makes async-signal-safe calls
+    // (the calling process may be multi-threaded, so the child must not allocate)
+    std::vector<char*> argv;
+    for (auto& a : args) argv.push_back(const_cast<char*>(a.c_str()));
+    argv.push_back(nullptr);
+    const int fd = open(log_path.c_str(), O_WRONLY | O_CREAT | O_TRUNC | O_CLOEXEC, 0644);
     pid_t pid = fork();
-    if (pid < 0) return fail(HRN_E_BUILD, "fork failed");
+    if (pid < 0) { if (fd >= 0) close(fd); return fail(HRN_E_BUILD, "fork failed"); }
     if (pid == 0) {
         setpgid(0, 0);
-        int fd = open(log_path.c_str(), O_WRONLY | O_CREAT | O_TRUNC, 0644);
-        if (fd >= 0) { dup2(fd, 1); dup2(fd, 2); close(fd); }
-        std::vector<char*> argv;
-        for (auto& a : args) argv.push_back(const_cast<char*>(a.c_str()));
-        argv.push_back(nullptr);
+        if (fd >= 0) { dup2(fd, 1); dup2(fd, 2); }
         execvp(argv[0], argv.data());
         _exit(127);
     }
+    if (fd >= 0) close(fd);
     auto t0 = std::chrono::steady_clock::now();
     int status = 0;
     for (;;) {
@@ -282,11 +286,11 @@ int compile_desc(const hrn_kernel_desc* d, double timeout_s, std::string* out_pa
     def("HRN_BKB", d->bkb); def("HRN_WM", d->wm); def("HRN_WN", d->wn); def("HRN_MFMA", d->mfma);
     def("HRN_STAGES", d->stages); def("HRN_SWZ", d->swizzle); def("HRN_EPI", d->epilogue);
     def("HRN_WPE", d->waves_per_eu);
-    def("HRN_ABLATE", d->ablate);   // diagnostic switches of the template, 0 in normal use
-    def("HRN_PF", d->l2_prefetch);
-    def("HRN_LOAD", d->load_mode);
     def("HRN_CONVWIN", d->conv_window);
     def("HRN_PERSIST", d->persistent);
+    def("HRN_SPLITK", d->split_k);
+    def("HRN_SCHED", d->sched);
+    def("HRN_LSPREAD", d->load_spread);
     {
         std::stringstream es(extra);
         std::string tok;
@@ -332,13 +336,37 @@ void read_info(const std::string& path, hrn_kernel_info* o) {
     }
 }
 
-int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, HrnKArgs* k,
-              unsigned* grid, unsigned* dyn_lds) {
-    *dyn_lds = 0;
+// What one launch consists of: the template kernel and, for a split-K instance, the pass that adds the K slices.
+struct LaunchPlan {
+    HrnKArgs k;
+    unsigned grid, dyn_lds;
+    int split;                 // K slices the grid covers (1 = the kernel writes C itself)
+    void* C;                   // the caller's output
+    int32_t ldc;
+    int64_t stride_c;
+};
+
+int64_t splitk_bytes(const hrn_problem* p, int split) { return (int64_t)split * p->batch * p->m * p->n * 4; }
+
+// k-tiles per slice and the number of non-empty slices for a requested split
+void split_shape(const hrn_kernel_desc& d, const hrn_problem* p, int* kt_per_slice, int* split) {
+    const int es = d.dtype == HRN_DT_F16 ? 2 : 1;
+    const int kt_all = (int)(((int64_t)p->k * es + d.bkb - 1) / d.bkb);
+    const int want = std::max(1, std::min(p->split_k, kt_all));
+    *kt_per_slice = (kt_all + want - 1) / want;
+    *split = (kt_all + *kt_per_slice - 1) / *kt_per_slice;
+}
+
+int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* workspace,
+              size_t workspace_bytes, LaunchPlan* plan) {
+    HrnKArgs* k = &plan->k;
+    plan->dyn_lds = 0;
+    plan->split = 1;
     if (!mod || !p || !A || !B || !C) return fail(HRN_E_BADPARAM, "null argument");
     const hrn_kernel_desc& d = mod->desc;
     if (p->op != d.op) return fail(HRN_E_BADPARAM, "problem op %d does not match module op %d", p->op, d.op);
     const int es = d.dtype == HRN_DT_F16 ? 2 : 1;
+    const int oes = d.dtype == HRN_DT_F16 ? 2 : 4;     // bytes of an element of the caller's C
     memset(k, 0, sizeof *k);
     k->A = A; k->B = B; k->C = C;
     if (p->m <= 0 || p->n <= 0 || p->k <= 0 || p->batch <= 0) return fail(HRN_E_BADPARAM, "empty problem");
@@ -348,10 +376,10 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
     k->lda = p->lda; k->ldb = p->ldb; k->ldc = p->ldc;
     k->sA = p->stride_a; k->sB = p->stride_b; k->sC = p->stride_c;
     k->batch = p->batch;
+    k->split = 1;
     if ((int64_t)p->ldb * es % 16 || p->ldb < p->k) return fail(HRN_E_BADPARAM, "ldb %d", p->ldb);
     if (p->ldc % 4 || p->ldc < p->n) return fail(HRN_E_BADPARAM, "ldc %d", p->ldc);
-    if (d.epilogue == 1 && (((int64_t)p->ldc * (d.dtype == HRN_DT_F16 ? 2 : 4)) % 16 || ((uintptr_t)C % 16) ||
-                            ((int64_t)p->stride_c * (d.dtype == HRN_DT_F16 ? 2 : 4)) % 16))
+    if (d.epilogue >= 1 && !d.split_k && (((int64_t)p->ldc * oes) % 16 || ((uintptr_t)C % 16) || ((int64_t)p->stride_c * oes) % 16))
         return fail(HRN_E_BADPARAM, "the LDS-staged epilogue stores 16 bytes per lane: C, ldc and stride_c must be 16-byte aligned");
     if ((int64_t)p->n * p->ldb * es >= (1ll << 31)) return fail(HRN_E_BADPARAM, "B operand exceeds 2 GiB per batch entry");
     if (d.op == HRN_OP_GEMM) {
@@ -379,23 +407,39 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
             if (p->kh * p->kw > 32) return fail(HRN_E_BADPARAM, "conv_window supports at most 32 filter taps");
             const int64_t rows = d.bm + 2 * ((int64_t)p->cpad * p->cw + p->cpad_w);
             const int64_t instr = (rows * (p->ci * es / 16) + 63) / 64;
-            const int64_t dyn = instr * 1024;
+            // dynamic LDS: the window, reused by the epilogue region (column sums, strips) once the last tap is read
+            const int64_t dyn = std::max<int64_t>(instr * 1024, mod->epi_bytes);
             if (dyn + mod->info.lds_bytes > 163840)
                 return fail(HRN_E_BADPARAM, "conv_window: window of %lld bytes + %d static LDS exceeds 163840", (long long)dyn, mod->info.lds_bytes);
-            *dyn_lds = (unsigned)dyn;
+            plan->dyn_lds = (unsigned)dyn;
         }
     }
     k->tiles_m = (p->m + d.bm - 1) / d.bm;
     k->tiles_n = (p->n + d.bn - 1) / d.bn;
     k->group_m = p->group_m > 0 ? p->group_m : 8;
-    // block of tiles one XCD (32 CUs) runs at a time under the kernel's raster: pf_sb rows x pf_sa columns
-    k->pf_sb = std::max(1, std::min(k->group_m, k->tiles_m));
-    k->pf_sa = std::max(1, std::min(k->tiles_n, 32 / k->pf_sb));
-    const int64_t total = (int64_t)k->tiles_m * k->tiles_n * p->batch;
+    int64_t total = (int64_t)k->tiles_m * k->tiles_n * p->batch;
+    plan->C = C; plan->ldc = p->ldc; plan->stride_c = p->stride_c;
+    if (d.split_k) {
+        // the kernel writes raw partial sums, slice by slice, into the workspace; hrn's reduction pass writes C
+        if (p->split_k < 1) return fail(HRN_E_BADPARAM, "a split_k instance needs problem.split_k >= 1 (got %d)", p->split_k);
+        int kps, split;
+        split_shape(d, p, &kps, &split);
+        const int64_t need = splitk_bytes(p, split);
+        if (!workspace || ((uintptr_t)workspace % 16)) return fail(HRN_E_BADPARAM, "split_k needs a 16-byte aligned device workspace");
+        if ((int64_t)workspace_bytes < need)
+            return fail(HRN_E_BADPARAM, "split_k workspace of %zu bytes is too small: %d slices x %d x %d x %d x 4 = %lld", workspace_bytes,
+                        split, p->batch, p->m, p->n, (long long)need);
+        if ((int64_t)p->m * p->n * 4 >= (1ll << 31)) return fail(HRN_E_BADPARAM, "split_k: one slice of C exceeds 2 GiB");
+        k->C = workspace; k->ldc = p->n; k->sC = (int64_t)p->m * p->n;
+        k->split = split; k->kt_per_slice = kps;
+        plan->split = split;
+        total *= split;
+    } else if (p->split_k > 1) {
+        return fail(HRN_E_BADPARAM, "problem.split_k = %d but the instance was not built with split_k", p->split_k);
+    }
     if (total <= 0 || total >= (1ll << 31)) return fail(HRN_E_BADPARAM, "grid size");
-    *grid = (unsigned)total;
+    plan->grid = (unsigned)total;
     if (d.persistent) {
-        const int oes = d.dtype == HRN_DT_F16 ? 2 : 4;
         if ((int64_t)p->n * oes % 16) return fail(HRN_E_BADPARAM, "persistent instances store whole 16-byte chunks: N*%d must be a multiple of 16", oes);
         if ((int64_t)p->m * p->ldc * oes >= (1ll << 31)) return fail(HRN_E_BADPARAM, "persistent: C exceeds 2 GiB per batch entry");
         int64_t g = std::min<int64_t>(total, mod->persist_grid);
@@ -404,22 +448,64 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
             if (v >= 1) g = std::min<int64_t>(total, v);
         }
         if (g >= 8) g &= ~7ll;          // workgroup i runs on XCD i % 8: keep tile t on XCD t % 8 in every round
-        *grid = (unsigned)g;
+        plan->grid = (unsigned)g;
+    }
+    return HRN_OK;
+}
+
+// Adds the K slices of a split-K launch: C[b,m,n] = sum_z ws[z,b,m,n], converted to the output type.  One lane per
+// 4 consecutive n (N is a multiple of 4): 16-byte reads, 8- or 16-byte writes.
+typedef float rv4f __attribute__((ext_vector_type(4)));
+typedef int rv4i __attribute__((ext_vector_type(4)));
+typedef _Float16 rv4h __attribute__((ext_vector_type(4)));
+
+template <bool F16>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const void* __restrict__ ws, void* __restrict__ C, int split,
+                                                            int batch, int M, int N, int ldc, int64_t stride_c) {
+    const int64_t n4 = N / 4;
+    const int64_t count = (int64_t)batch * M * n4;
+    const int64_t slice = (int64_t)batch * M * N;           // elements of one slice
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t bm = i / n4;
+        const int q = (int)(i - bm * n4);
+        const int b = (int)(bm / M), m = (int)(bm - (int64_t)b * M);
+        const int64_t src = bm * N + (int64_t)q * 4;
+        const int64_t dst = (int64_t)b * stride_c + (int64_t)m * ldc + (int64_t)q * 4;
+        if constexpr (F16) {
+            rv4f acc = *(const rv4f*)((const float*)ws + src);
+            for (int z = 1; z < split; ++z) acc += *(const rv4f*)((const float*)ws + z * slice + src);
+            rv4h o;
+            for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[r];
+            *(rv4h*)((_Float16*)C + dst) = o;
+        } else {
+            rv4i acc = *(const rv4i*)((const int*)ws + src);
+            for (int z = 1; z < split; ++z) acc += *(const rv4i*)((const int*)ws + z * slice + src);
+            *(rv4i*)((int*)C + dst) = acc;
+        }
+    }
+}
+
+int run_plan(const hrn_module* mod, const hrn_problem* p, const LaunchPlan& plan, void* workspace, hipStream_t st) {
+    size_t sz = sizeof plan.k;
+    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, (void*)&plan.k, HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
+    HIP_TRY(hipModuleLaunchKernel(mod->fn, plan.grid, 1, 1, (unsigned)mod->info.threads, 1, 1, plan.dyn_lds, st, nullptr, extra));
+    if (mod->desc.split_k) {
+        const int64_t count = (int64_t)p->batch * p->m * (p->n / 4);
+        const unsigned blocks = (unsigned)std::min<int64_t>((count + 255) / 256, 256 * 32);
+        if (mod->desc.dtype == HRN_DT_F16)
+            splitk_reduce_kernel<true><<<blocks, 256, 0, st>>>(workspace, plan.C, plan.split, p->batch, p->m, p->n, plan.ldc, plan.stride_c);
+        else
+            splitk_reduce_kernel<false><<<blocks, 256, 0, st>>>(workspace, plan.C, plan.split, p->batch, p->m, p->n, plan.ldc, plan.stride_c);
+        HIP_TRY(hipGetLastError());
     }
     return HRN_OK;
 }
 
 int launch(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream) {
-    HrnKArgs k;
-    unsigned grid;
-    unsigned dyn_lds;
-    int rc = fill_args(mod, p, A, B, C, &k, &grid, &dyn_lds);
+    LaunchPlan plan;
+    int rc = fill_args(mod, p, A, B, C, p ? p->workspace : nullptr, p ? p->workspace_bytes : 0, &plan);
     if (rc) return rc;
-    size_t sz = sizeof k;
-    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &k, HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
-    HIP_TRY(hipModuleLaunchKernel(mod->fn, grid, 1, 1, (unsigned)mod->info.threads, 1, 1, dyn_lds, (hipStream_t)stream,
-                                  nullptr, extra));
-    return HRN_OK;
+    return run_plan(mod, p, plan, p->workspace, (hipStream_t)stream);
 }
 
 // ---- roofline probes -----------------------------------------------------------------------
@@ -472,7 +558,8 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(float* sink, int iters,
         }
         float s = 0;
         for (int r = 0; r < 16; ++r) s += (float)(c0[r] + c1[r] + c2[r] + c3[r]);
-        if (s == 123.456f) sink[0] = s;
+        asm volatile("" ::"v"(s));   // keeps the accumulators live; nothing is stored
+        (void)sink;
     } else {
         using acc_t = typename std::conditional<KIND == 1, pv4f, pv4i>::type;
         acc_t c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
@@ -491,7 +578,8 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(float* sink, int iters,
         }
         float s = 0;
         for (int r = 0; r < 4; ++r) s += (float)(c0[r] + c1[r] + c2[r] + c3[r]);
-        if (s == 123.456f) sink[0] = s;
+        asm volatile("" ::"v"(s));   // keeps the accumulators live; nothing is stored
+        (void)sink;
     }
 }
 
@@ -626,6 +714,11 @@ int hrn_build(const hrn_kernel_desc* desc, double timeout_s, hrn_module** out) {
     memset(&m->info, 0, sizeof m->info);
     read_info(path.substr(0, path.size() - 6) + ".info", &m->info);
     m->info.threads = desc->wm * desc->wn * 64;
+    {
+        Derived dv;
+        (void)derive(desc, &dv);        // compile_desc has validated the descriptor
+        m->epi_bytes = dv.epi_bytes;
+    }
     hipError_t e = hipModuleLoad(&m->mod, path.c_str());
     if (e != hipSuccess) {
         delete m;
@@ -700,26 +793,21 @@ int hrn_launch_conv2d_nhwc_u8s8(const hrn_module* mod, const hrn_problem* p, con
 int hrn_launch_repeat(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, int count,
                       void* stream) {
     if (count < 1) return fail(HRN_E_BADPARAM, "count %d", count);
-    HrnKArgs k;
-    unsigned grid;
-    unsigned dyn_lds;
-    int rc = fill_args(mod, p, A, B, C, &k, &grid, &dyn_lds);
+    LaunchPlan plan;
+    int rc = fill_args(mod, p, A, B, C, p ? p->workspace : nullptr, p ? p->workspace_bytes : 0, &plan);
     if (rc) return rc;
-    size_t sz = sizeof k;
-    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &k, HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
-    for (int i = 0; i < count; ++i)
-        HIP_TRY(hipModuleLaunchKernel(mod->fn, grid, 1, 1, (unsigned)mod->info.threads, 1, 1, dyn_lds, (hipStream_t)stream,
-                                      nullptr, extra));
+    for (int i = 0; i < count; ++i) {
+        rc = run_plan(mod, p, plan, p->workspace, (hipStream_t)stream);
+        if (rc) return rc;
+    }
     return HRN_OK;
 }
 
 int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, int number, int repeat,
              double min_repeat_ms, double* costs_out, void* stream) {
     if (!costs_out || number < 1 || repeat < 1) return fail(HRN_E_BADPARAM, "number/repeat/costs_out");
-    HrnKArgs k;
-    unsigned grid;
-    unsigned dyn_lds;
-    int rc = fill_args(mod, p, A, B, C, &k, &grid, &dyn_lds);
+    LaunchPlan plan;
+    int rc = fill_args(mod, p, A, B, C, p ? p->workspace : nullptr, p ? p->workspace_bytes : 0, &plan);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
     EventPair ev;
@@ -756,10 +844,8 @@ int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const v
 int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* flush_buf,
                   size_t flush_bytes, int repeat, double* costs_out, void* stream) {
     if (!costs_out || repeat < 1 || !flush_buf || flush_bytes < (64u << 20)) return fail(HRN_E_BADPARAM, "repeat/costs_out/flush buffer (>= 64 MiB)");
-    HrnKArgs k;
-    unsigned grid;
-    unsigned dyn_lds;
-    int rc = fill_args(mod, p, A, B, C, &k, &grid, &dyn_lds);
+    LaunchPlan plan;
+    int rc = fill_args(mod, p, A, B, C, p ? p->workspace : nullptr, p ? p->workspace_bytes : 0, &plan);
     if (rc) return rc;
     int dev = 0;
     hipDeviceProp_t pr;
@@ -785,6 +871,16 @@ int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, co
         costs_out[r] = (double)ms * 1e-3;
     }
     return HRN_OK;
+}
+
+int64_t hrn_splitk_workspace_bytes(const hrn_kernel_desc* desc, const hrn_problem* p) {
+    if (!desc || !p) return fail(HRN_E_BADPARAM, "null argument");
+    if (!desc->split_k) return 0;
+    if (p->m <= 0 || p->n <= 0 || p->k <= 0 || p->batch <= 0 || p->split_k < 1) return fail(HRN_E_BADPARAM, "empty problem or split_k < 1");
+    if (desc->bkb != 64 && desc->bkb != 128 && desc->bkb != 256) return fail(HRN_E_BADPARAM, "bkb %d", desc->bkb);
+    int kps, split;
+    split_shape(*desc, p, &kps, &split);
+    return splitk_bytes(p, split);
 }
 
 void hrn_problem_gemm(hrn_problem* p, int batch, int m, int n, int k) {

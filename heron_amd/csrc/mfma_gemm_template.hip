@@ -8,19 +8,23 @@
 //   HRN_BM/BN   workgroup tile, HRN_BKB bytes of K per LDS row, HRN_WM x HRN_WN wave grid,
 //   HRN_MFMA    32 | 16 (MFMA tile edge), HRN_STAGES LDS stages, HRN_SWZ LDS chunk swizzle,
 //   HRN_EPI     0 stores straight from the accumulator registers, 1 LDS-staged epilogue with 16-byte coalesced
-//               stores, HRN_WPE waves-per-SIMD hint, HRN_PF L2 prefetch distance, HRN_LOAD load path.
+//               stores, 2 the same with half-width staging strips, HRN_WPE waves-per-SIMD hint, HRN_CONVWIN conv input window in LDS, HRN_PERSIST persistent
+//               launch, HRN_SPLITK K split over several workgroups with raw partial sums as output.
 //
 // Data movement: both operands are K-contiguous, so a tile is a set of rows of HRN_BKB bytes.
 // Rows are cut into 16-byte chunks; every lane moves one chunk per load straight from HBM/L2
 // into LDS (buffer_load_dwordx4 ... lds), one wave instruction filling 1 KiB of consecutive LDS.
 // The chunk a lane fetches is XOR-swizzled so that the MFMA operand reads (ds_read_b128, one
-// 16-byte chunk per lane) spread over all LDS banks.  Out-of-range rows, conv halo taps and the
-// dummy tiles past the end of K are fetched with an out-of-range buffer offset, which the
-// buffer unit turns into zeros.
+// 16-byte chunk per lane) spread over all LDS banks.  A lane's byte offset inside its row never
+// changes; the k-tile is selected by the scalar offset operand of the load, so the k-loop spends
+// no vector instruction on addresses.  Out-of-range rows and conv halo taps are fetched with an
+// out-of-range lane offset, the dummy tiles past the end of K through a zero-length buffer
+// descriptor: the buffer unit turns both into zeros.
 //
 // Pipeline: HRN_STAGES tiles are in flight.  The barrier that publishes tile t+1 sits before the
 // last k-step of tile t, so operand fragments of the next tile are already being read while the
-// last MFMAs of the current tile run; fragments are double-buffered in registers.
+// last MFMAs of the current tile run; fragments are double-buffered in registers and read in the
+// order the MFMAs of the next step consume them (all of B, then A row-tile by row-tile).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <type_traits>
@@ -41,8 +45,8 @@ struct HrnKArgs {
     int32_t tiles_m, tiles_n, group_m, batch;
     // conv
     int32_t H, W, CI, HO, WO, KH, KW, cstride, cpad, cdil;
-    int32_t pf_sa, pf_sb;       // L2 prefetch: column-tiles / row-tiles of the block one XCD runs concurrently
     int32_t cstride_w, cpad_w, cdil_w;   // conv: the width-direction values (cstride/cpad/cdil are the height ones)
+    int32_t split, kt_per_slice;         // split-K: number of K slices and k-tiles per slice
 };
 #endif
 
@@ -53,34 +57,18 @@ constexpr int OP = HRN_OP;
 constexpr int BM = HRN_BM, BN = HRN_BN, BKB = HRN_BKB;
 constexpr int WM = HRN_WM, WN = HRN_WN, MT = HRN_MFMA, NS = HRN_STAGES, SWZ = HRN_SWZ;
 constexpr int EPI = HRN_EPI;
-// Diagnostic switches for bottleneck analysis (results are WRONG when non-zero; 0 in every shipped
-// instance): 1 skip LDS fragment reads after the first tile, 2 skip global->LDS loads after the
-// prologue, 4 drop the per-tile barrier, 8 skip the MFMAs, 16 skip the stores of C.
+// Study switches for bottleneck analysis, set only through extra compiler flags (results are WRONG when non-zero):
+// 1 skip LDS fragment reads after the first tile, 2 skip global->LDS loads after the prologue, 4 drop the per-tile
+// barrier, 8 skip the MFMAs, 16 skip the stores of C.
 #ifndef HRN_ABLATE
 #define HRN_ABLATE 0
 #endif
 constexpr int ABL = HRN_ABLATE;
-// L2 prefetch: with HRN_PF = d > 0 every tile fetch is preceded by 4-byte "touch" loads of the k-tile d tiles
-// further on (this workgroup's share of the rows, see the kernel).  The data is discarded; the point is that
-// the sectors are in L2 (not HBM) when the real fetch arrives, because a tile is only usable when its slowest
-// load has landed.
-#ifndef HRN_PF
-#define HRN_PF 0
-#endif
-constexpr int PF = HRN_PF;
-// Load path: 0 = global -> LDS directly (LDS-DMA), HRN_STAGES tiles in LDS.
-//            1 = global -> registers -> LDS: two register sets hold the two tiles in flight, LDS holds the tile
-//                being multiplied and the next one (HRN_STAGES must be 2); a tile then has two tile-times to land.
-#ifndef HRN_LOAD
-#define HRN_LOAD 0
-#endif
-
-constexpr int LOADM = HRN_LOAD;
 // Conv window mode (HRN_OP=1, stride 1, dilation 1, 'same' padding): instead of fetching an im2col tile of A for every
 // filter tap, the workgroup loads ONCE the window of input pixels its BM output pixels can reach (a contiguous range
 // of BM + 2*(pad_h*W + pad_w) pixels, all channels) and every tap reads its operand fragments from that window at a row offset
 // of r*W + s pixels; taps that fall into the padding are masked to zero in registers.  Only B (the filter) streams
-// through the LDS stages.
+// through the LDS stages.  The window lives in dynamic LDS; the staged epilogue reuses it once the last tap is read.
 #ifndef HRN_CONVWIN
 #define HRN_CONVWIN 0
 #endif
@@ -95,16 +83,31 @@ constexpr bool CW = (HRN_CONVWIN != 0);
 #define HRN_PERSIST 0
 #endif
 constexpr bool PERS = (HRN_PERSIST != 0);
-constexpr int ES = (DT == 0) ? 2 : 1;       // input element bytes
-constexpr int OES = (DT == 0) ? 2 : 4;      // output element bytes
+// Split-K: the grid holds `split` copies of the tile grid; copy z multiplies k-tiles [z*kt_per_slice, (z+1)*kt_per_slice)
+// and stores its raw fp32 / int32 partial sums to slice z of the output buffer (a workspace); a second kernel adds the slices.
+#ifndef HRN_SPLITK
+#define HRN_SPLITK 0
+#endif
+constexpr bool SPLITK = (HRN_SPLITK != 0);
+// Issue order of a k-step: 1 = the source order of the row groups is pinned (a scheduling fence after every row of
+// MFMAs), 0 = the compiler interleaves on its own, guided by group hints (one LDS read per few MFMAs).
+#ifndef HRN_SCHED
+#define HRN_SCHED 1
+#endif
+constexpr int SCHED = HRN_SCHED;
+#ifndef HRN_LSPREAD
+#define HRN_LSPREAD 2
+#endif
+constexpr int LSPREAD = HRN_LSPREAD;
+static_assert(LSPREAD >= 0 && LSPREAD <= 3, "load spread");
+constexpr int ES = (DT == 0) ? 2 : 1;                  // input element bytes
+constexpr int OES = (DT == 0 && !SPLITK) ? 2 : 4;      // output element bytes
 constexpr int NW = WM * WN, NT = NW * 64;
 constexpr int CPR = BKB / 16;               // 16-byte chunks per tile row
 constexpr int RPI = 64 / CPR;               // tile rows one wave load instruction covers
 constexpr int A_LPW = CW ? 0 : (BM / RPI) / NW;   // load instructions per wave per tile
 constexpr int B_LPW = (BN / RPI) / NW;
-constexpr int LPR = (BKB + 127) / 128;                         // 128-byte lines per tile row
-constexpr int PF_N = PF ? 1 : 0;                                // prefetch touches per lane per tile
-constexpr int LPT = A_LPW + B_LPW + PF_N;                       // vector memory ops per lane per tile
+constexpr int LPT = A_LPW + B_LPW;          // vector memory ops per lane per tile
 constexpr int KSB = (MT == 32) ? 32 : 64;   // bytes of K one MFMA consumes
 constexpr int KS = BKB / KSB;               // MFMA k-steps per tile
 constexpr int CPS = KSB / 16;               // chunks per k-step (= 64 / MT)
@@ -116,31 +119,36 @@ constexpr uint32_t OOB = 0x80000000u;
 
 static_assert(BKB == 64 || BKB == 128 || BKB == 256, "BKB");
 static_assert(MT == 32 || MT == 16, "MFMA");
-static_assert(KS >= 2 && (KS % 2) == 0, "need an even number of k-steps per tile");
+static_assert(KS >= 1, "k-steps per tile");
+static_assert((WM & (WM - 1)) == 0, "wave rows must be a power of two");
 static_assert((CW || ((BM / RPI) % NW == 0 && A_LPW >= 1)) && (BN / RPI) % NW == 0 && B_LPW >= 1, "loads per wave");
-static_assert(!CW || (OP == 1 && LOADM == 0 && PF == 0), "window mode is a conv2d load path");
-static_assert(OP == 0 || PF == 0, "L2 prefetch is implemented for the GEMM address pattern only");
-static_assert(PF == 0 || NW >= 2, "L2 prefetch needs one wave for each operand");
+static_assert(!CW || OP == 1, "window mode is a conv2d load path");
 static_assert(BM % (WM * MT) == 0 && BN % (WN * MT) == 0, "wave tile");
 static_assert(NS >= 2 && NS <= 5, "stages");
-static_assert(LOADM == 0 || (NS == 2 && PF == 0), "register-staged loads use exactly two LDS stages");
-constexpr int PF_SCRATCH = PF ? NW * 256 : 0;                   // LDS corner the prefetch touches land in
-// LDS-staged epilogue: per wave a strip of MT rows x WTN outputs, rows padded by 16 bytes; after the int8 column sums
-constexpr int EPI_PITCH = WTN * OES + 16;
-constexpr int EPI_BASE = (DT == 1) ? ((BN * 4 + 1023) / 1024) * 1024 : 0;
-constexpr int EPI_BYTES = (EPI == 1) ? EPI_BASE + NW * MT * EPI_PITCH : 0;
-// the epilogue region (column sums + strips) reuses the stages, except in persistent mode where the stages stay live
+// LDS-staged epilogue: per wave a strip of MT rows x WTN outputs, rows padded by 16 bytes; in front of the strips the
+// uint8 path keeps the column sums of B, one row of BN sums per wave row (each wave row sums its share of the k-steps)
+// (HRN_EPI = 2: strips of half the wave tile's width, filled and written out twice per row-tile - half the LDS)
+constexpr int ESPLIT = (EPI == 2) ? 2 : 1;
+constexpr int SW = WTN / ESPLIT;            // outputs per strip row
+constexpr int EPI_PITCH = SW * OES + 16;
+constexpr int EPI_BASE = (DT == 1) ? ((WM * BN * 4 + 1023) / 1024) * 1024 : 0;
+constexpr int EPI_BYTES = (EPI >= 1) ? EPI_BASE + NW * MT * EPI_PITCH : 0;
+// the epilogue region (column sums + strips) reuses the stages (window mode: the window), except in persistent mode
+// where the stages stay live
 constexpr int EPI_OFF = PERS ? NS * STAGE_BYTES : 0;
 constexpr int LDS_BYTES = PERS ? NS * STAGE_BYTES + EPI_BYTES
-                               : ((NS * STAGE_BYTES + PF_SCRATCH > EPI_BYTES) ? NS * STAGE_BYTES + PF_SCRATCH : EPI_BYTES);
-constexpr int STORES_PER_TILE = (EPI == 1) ? TM * (MT * (WTN * OES / 16) / 64) : 0;   // store instructions per wave per output tile
-static_assert(!PERS || (EPI == 1 && LOADM == 0 && PF == 0 && !CW && HRN_ABLATE == 0), "persistent mode: staged epilogue, direct loads");
-static_assert(!PERS || (NS - 2) * (A_LPW + B_LPW) + STORES_PER_TILE <= 63, "persistent mode: vmcnt range");
+                               : ((CW || NS * STAGE_BYTES > EPI_BYTES) ? NS * STAGE_BYTES : EPI_BYTES);
+constexpr int STORES_PER_TILE = (EPI >= 1) ? TM * ESPLIT * (MT * (SW * OES / 16) / 64) : 0;   // store instructions per wave per output tile
+static_assert(EPI >= 0 && EPI <= 2 && TN % ESPLIT == 0, "epilogue kind");
+static_assert(!PERS || (EPI >= 1 && !CW && !SPLITK && HRN_ABLATE == 0 && KS % 2 == 0), "persistent mode: staged epilogue, even k-steps");
+static_assert(!PERS || (NS - 2) * LPT + STORES_PER_TILE <= 63, "persistent mode: vmcnt range");
+static_assert(!SPLITK || !CW, "split-K uses the im2col load path");
 static_assert(LDS_BYTES <= 163840, "LDS");
-static_assert(EPI == 0 || (MT * (WTN * OES / 16)) % 64 == 0, "staged epilogue: a strip must split into whole wave stores");
+static_assert(EPI == 0 || (MT * (SW * OES / 16)) % 64 == 0, "staged epilogue: a strip must split into whole wave stores");
 static_assert(SWZ == 0 || (CPR << (SWZ - 1)) <= MT, "swizzle period must fit in one MFMA tile");
 static_assert((NS - 1) * LPT <= 63, "vmcnt range");
 static_assert(NT <= 1024, "threads");
+static_assert(DT == 0 || NS * STAGE_BYTES >= WM * BN * 4, "column sums must fit the stages");
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -176,14 +184,15 @@ __device__ __forceinline__ void wait_only() {
 
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
-// raw buffer (stride 0): an offset >= `bytes` reads as zero instead of touching memory
+// raw buffer (stride 0): a lane offset >= `bytes` reads as zero instead of touching memory (the scalar offset of a
+// load is not part of that check)
 __device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
 
-__device__ __forceinline__ void load_chunk_to_lds(rsrc_t rsrc, char* lds_wave_base, uint32_t voff) {
+__device__ __forceinline__ void load_chunk_to_lds(rsrc_t rsrc, char* lds_wave_base, uint32_t voff, uint32_t soff) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds_wave_base,
-                                             16, (int)voff, 0, 0, 0);
+                                             16, (int)voff, (int)soff, 0, 0);
 }
 
 __device__ __forceinline__ v16f mfma(v4i x, v4i y, v16f c) {
@@ -199,18 +208,16 @@ __device__ __forceinline__ v4i mfma(v4i x, v4i y, v4i c) {
     return __builtin_amdgcn_mfma_i32_16x16x64_i8(x, y, c, 0, 0, 0);
 }
 
-// Scheduling pattern of one k-step: NR groups of {1 LDS read, NV/NR buffer loads, NDW/NR LDS writes, NMM/NR MFMAs}.
-template <int R, int NR, int NMM, int NV, int NDW = 0>
-__device__ __forceinline__ void sched_pattern() {
+// Scheduling hints of one k-step (HRN_SCHED = 0): NR groups of {1 LDS read, NV/NR buffer loads, NMM/NR MFMAs}.
+template <int R, int NR, int NMM, int NV>
+__device__ __forceinline__ void sched_hint() {
     if constexpr (R < NR) {
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         constexpr int v = (NV * (R + 1)) / NR - (NV * R) / NR;
         if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);
-        constexpr int w = (NDW * (R + 1)) / NR - (NDW * R) / NR;
-        if constexpr (w > 0) __builtin_amdgcn_sched_group_barrier(0x200, w, 0);
         constexpr int mm = (NMM * (R + 1)) / NR - (NMM * R) / NR;
         if constexpr (mm > 0) __builtin_amdgcn_sched_group_barrier(0x008, mm, 0);
-        sched_pattern<R + 1, NR, NMM, NV, NDW>();
+        sched_hint<R + 1, NR, NMM, NV>();
     }
 }
 
@@ -222,6 +229,7 @@ __attribute__((amdgpu_waves_per_eu(HRN_WPE, HRN_WPE)))
 #endif
 hrn_mfma_kernel(const HrnKArgs a) {
     __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+    extern __shared__ __attribute__((aligned(1024))) char win[];   // window mode: input window, later the epilogue region
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -229,27 +237,31 @@ hrn_mfma_kernel(const HrnKArgs a) {
     const int wm_idx = wave / WN, wn_idx = wave % WN;
 
     const int tiles_mn = a.tiles_m * a.tiles_n;
-    const int total = tiles_mn * a.batch;
+    const int total = tiles_mn * a.batch;             // output tiles (of one K slice)
     const uint32_t Kb = (uint32_t)a.K * ES;           // bytes of K
-    const int KT = (Kb + BKB - 1) / BKB;
+    const int KT_all = (Kb + BKB - 1) / BKB;
+    int first_pid = blockIdx.x, slice = 0;
+    if constexpr (SPLITK) { slice = first_pid / total; first_pid -= slice * total; }
+    const int kt0 = SPLITK ? slice * a.kt_per_slice : 0;                                   // first k-tile of this workgroup
+    const int KT = SPLITK ? min(a.kt_per_slice, KT_all - kt0) : KT_all;                    // k-tiles of this workgroup
 
     // ---- tile raster: spread over the 8 XCDs so that each XCD's L2 sees a compact block ----
-    auto tile_coords = [&](int pid, int& bz, int& tile_m, int& tile_n, int& tin, int& gsz) {
+    auto tile_coords = [&](int pid, int& bz, int& tile_m, int& tile_n) {
         if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
         bz = pid / tiles_mn;
         const int t = pid - bz * tiles_mn;
         const int group_sz = a.group_m * a.tiles_n;
         const int gid = t / group_sz;
         const int first_m = gid * a.group_m;
-        gsz = min(a.tiles_m - first_m, a.group_m);
-        tin = t - gid * group_sz;
+        const int gsz = min(a.tiles_m - first_m, a.group_m);
+        const int tin = t - gid * group_sz;
         tile_m = first_m + tin % gsz;
         tile_n = tin / gsz;
     };
 
     // ---- compute side: the output tile whose accumulators this workgroup holds ----
-    int c_bz, c_tile_m, c_tile_n, c_tin, c_gsz;
-    tile_coords(blockIdx.x, c_bz, c_tile_m, c_tile_n, c_tin, c_gsz);
+    int c_bz, c_tile_m, c_tile_n;
+    tile_coords(first_pid, c_bz, c_tile_m, c_tile_n);
     int m0 = c_tile_m * BM, n0 = c_tile_n * BN;
 
     // ---- issue side: the tile whose k-tiles are being fetched (the same tile unless the launch is persistent) ----
@@ -257,8 +269,9 @@ hrn_mfma_kernel(const HrnKArgs a) {
     const uint32_t b_bytes = (uint32_t)a.N * (uint32_t)a.ldb * ES;
     if constexpr (OP == 0) a_bytes = (uint32_t)a.M * (uint32_t)a.lda * ES;
     else a_bytes = (uint32_t)(a.M / (a.HO * a.WO)) * (uint32_t)(a.H * a.W * a.CI) * ES;
-    rsrc_t rsrcA = make_rsrc(a.A, a_bytes);
-    rsrc_t rsrcB = make_rsrc(a.B, b_bytes);
+    const char* baseA = (const char*)a.A;
+    const char* baseB = (const char*)a.B;
+    bool issue_alive = true;
 
     const int lrow = lane / CPR, lpos = lane % CPR;
     uint32_t voffB[B_LPW];
@@ -266,22 +279,22 @@ hrn_mfma_kernel(const HrnKArgs a) {
     uint32_t voffA[(A_LPW > 0 ? A_LPW : 1)];
     int iy0[OP == 1 ? (A_LPW > 0 ? A_LPW : 1) : 1], ix0[OP == 1 ? (A_LPW > 0 ? A_LPW : 1) : 1];
     int cc = 0, cs = 0, cr = 0;  // conv: channel / kw / kh position of the lane's chunk
-    int itile = blockIdx.x;
-    int issue_kt = 0;            // next k-tile of tile `itile` to fetch
+    int itile = first_pid;
+    int issue_kt = 0;            // next k-tile (relative to kt0) of tile `itile` to fetch
 
     auto setup_issue = [&](int t) {
-        const bool alive = t < total;                 // past the last tile every fetch reads zeros
-        int bz, tile_m, tile_n, tin, gsz;
-        tile_coords(alive ? t : 0, bz, tile_m, tile_n, tin, gsz);
+        issue_alive = t < total;                      // past the last tile every fetch reads zeros
+        int bz, tile_m, tile_n;
+        tile_coords(issue_alive ? t : 0, bz, tile_m, tile_n);
         const int im0 = tile_m * BM, in0 = tile_n * BN;
-        rsrcA = make_rsrc((const char*)a.A + (int64_t)bz * a.sA * ES, a_bytes);
-        rsrcB = make_rsrc((const char*)a.B + (int64_t)bz * a.sB * ES, b_bytes);
+        baseA = (const char*)a.A + (int64_t)bz * a.sA * ES;
+        baseB = (const char*)a.B + (int64_t)bz * a.sB * ES;
 #pragma unroll
         for (int i = 0; i < B_LPW; ++i) {
             const int row = (i * NW + wave) * RPI + lrow;
             const int chunk = lpos ^ swz_of_row(row);
             const int n = in0 + row;
-            voffB[i] = (alive && n < a.N) ? (uint32_t)n * (uint32_t)a.ldb * ES + chunk * 16 : OOB;
+            voffB[i] = (n < a.N) ? (uint32_t)n * (uint32_t)a.ldb * ES + chunk * 16 : OOB;
         }
         if constexpr (OP == 0) {
 #pragma unroll
@@ -289,13 +302,13 @@ hrn_mfma_kernel(const HrnKArgs a) {
                 const int row = (i * NW + wave) * RPI + lrow;
                 const int chunk = lpos ^ swz_of_row(row);
                 const int m = im0 + row;
-                voffA[i] = (alive && m < a.M) ? (uint32_t)m * (uint32_t)a.lda * ES + chunk * 16 : OOB;
+                voffA[i] = (m < a.M) ? (uint32_t)m * (uint32_t)a.lda * ES + chunk * 16 : OOB;
             }
         } else if constexpr (!CW) {
-            static_assert(OP == 0 || SWZ == 0 || ((NW * RPI) % (CPR << (SWZ > 0 ? SWZ - 1 : 0))) == 0,
+            static_assert(OP == 0 || CW || SWZ == 0 || ((NW * RPI) % (CPR << (SWZ > 0 ? SWZ - 1 : 0))) == 0,
                           "conv: the lane's chunk column must not depend on the load index");
             const int chunk = lpos ^ swz_of_row(wave * RPI + lrow);
-            int ke = chunk * (16 / ES);                 // element index inside K of tile 0
+            int ke = chunk * (16 / ES) + kt0 * (BKB / ES);      // element index inside K of this workgroup's first k-tile
             cr = ke / (a.KW * a.CI); ke -= cr * (a.KW * a.CI);
             cs = ke / a.CI; cc = ke - cs * a.CI;
             // output pixel of the lane's first row by division, of the following rows (NW*RPI further each) by carry
@@ -306,7 +319,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
             int oy = rem / a.WO, ox = rem - oy * a.WO;
 #pragma unroll
             for (int i = 0; i < A_LPW; ++i) {
-                const bool ok = alive && m < a.M;
+                const bool ok = m < a.M;
                 voffA[i] = (uint32_t)img * (uint32_t)(a.H * a.W * a.CI) * ES;
                 iy0[i] = ok ? oy * a.cstride - a.cpad : -(1 << 28);
                 ix0[i] = ox * a.cstride_w - a.cpad_w;
@@ -318,65 +331,6 @@ hrn_mfma_kernel(const HrnKArgs a) {
     };
     setup_issue(itile);
 
-    // L2 prefetch duty of this workgroup.  The tiles that run on one XCD at the same time form a block of
-    // a.pf_sb row-tiles x a.pf_sa column-tiles; the pf_sa tiles of one block row read the same rows of A and the
-    // pf_sb tiles of one block column the same rows of B, so each tile touches only its 1/pf_sa share of the A rows
-    // and 1/pf_sb share of the B rows (every 64-byte sector of them) of the k-tile PF tiles past the one being
-    // fetched.  Waves of the lower half touch A, waves of the upper half B, one touch per lane per tile.
-    uint32_t pf_off[PF_N > 0 ? PF_N : 1];
-    const bool pf_isb = wave >= (NW + 1) / 2;
-    if constexpr (PF > 0) {
-        constexpr int SEC = BKB >= 64 ? BKB / 64 : 1;
-        const int share = pf_isb ? a.pf_sb : a.pf_sa;
-        const int duty = pf_isb ? (c_tin % c_gsz) % share : c_tile_n % share;
-        const int q = (pf_isb ? tid - ((NW + 1) / 2) * 64 : tid);      // touch slot inside the operand's waves
-        const int row = duty + share * (q / SEC), sec = q % SEC;
-        const int g = (pf_isb ? n0 : m0) + row;
-        const bool ok = row < (pf_isb ? BN : BM) && g < (pf_isb ? a.N : a.M);
-        pf_off[0] = ok ? (uint32_t)g * (uint32_t)(pf_isb ? a.ldb : a.lda) * ES + sec * 64 : OOB;
-    }
-
-    // Byte offsets of this lane's chunks in k-tile `issue_kt` (out-of-range offset = zeros), shared by both load paths.
-    uint32_t offA[(A_LPW > 0 ? A_LPW : 1)], offB[B_LPW];
-    auto tile_offsets = [&]() {
-        const bool live = issue_kt < KT;
-        const bool ragged = (uint32_t)(issue_kt + 1) * BKB > Kb;   // last tile not full (wave-uniform)
-        const uint32_t koff = live ? (uint32_t)issue_kt * BKB : OOB;
-        if constexpr (OP == 0) {
-#pragma unroll
-            for (int i = 0; i < A_LPW; ++i) {
-                uint32_t v = voffA[i] + koff;
-                if (ragged && live) {
-                    const int row = (i * NW + wave) * RPI + lrow;
-                    const uint32_t kb = koff + (uint32_t)((lpos ^ swz_of_row(row)) * 16);
-                    if (kb >= Kb) v = OOB;
-                }
-                offA[i] = v;
-            }
-        } else if constexpr (!CW) {
-            const int iyr = cr * a.cdil, ixs = cs * a.cdil_w;
-            const bool kvalid = live && cr < a.KH;
-#pragma unroll
-            for (int i = 0; i < A_LPW; ++i) {
-                const int iy = iy0[i] + iyr, ix = ix0[i] + ixs;
-                const bool ok = kvalid && (unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W;
-                offA[i] = ok ? voffA[i] + (uint32_t)((iy * a.W + ix) * a.CI + cc) * ES : OOB;
-            }
-            // advance the lane's (kh, kw, ci) position by one k-tile
-            cc += BKB / ES;
-            while (cc >= a.CI) { cc -= a.CI; if (++cs == a.KW) { cs = 0; ++cr; } }
-        }
-#pragma unroll
-        for (int i = 0; i < B_LPW; ++i) {
-            uint32_t v = voffB[i] + koff;
-            if (ragged && live) {
-                const int row = (i * NW + wave) * RPI + lrow;
-                const uint32_t kb = koff + (uint32_t)((lpos ^ swz_of_row(row)) * 16);
-                if (kb >= Kb) v = OOB;
-            }
-            offB[i] = v;
-        }
-    };
     // the stream moves on: next k-tile of this tile, or (persistent) k-tile 0 of the workgroup's next tile
     auto advance_issue = [&]() {
         ++issue_kt;
@@ -385,56 +339,88 @@ hrn_mfma_kernel(const HrnKArgs a) {
         }
     };
 
-    // path 0: fetch k-tile `issue_kt` straight into LDS stage `stage`
-    auto issue_tile = [&](int stage) {
+    // Fetch k-tile `issue_kt` of the issue-side tile straight into LDS stage `stage`: begin_issue() fixes the tile's
+    // descriptors and scalar offset, issue_loads(first, count) emits a part of its LPT wave loads (A first, then B), so
+    // that the caller can spread them between MFMAs, end_issue() moves the stream on.  RAG = the tile may be the last,
+    // partly filled one (its chunks past the end of K are masked per lane); the plain form spends no vector ALU work.
+    rsrc_t rA_cur, rB_cur;
+    uint32_t ks_cur = 0, koff_cur = 0;
+    auto begin_issue = [&]() {
+        const bool live = issue_alive && issue_kt < KT;                          // wave-uniform
+        koff_cur = (uint32_t)(kt0 + issue_kt) * BKB;                             // byte offset of the k-tile in a row
+        // a dead tile (past the end of K, or past the workgroup's last output tile) reads zeros through empty descriptors
+        rB_cur = make_rsrc(baseB, live ? b_bytes : 0u);
+        rA_cur = make_rsrc(baseA, live ? a_bytes : 0u);
+        ks_cur = live ? koff_cur : 0u;
+        return live && koff_cur + BKB > Kb;                                      // ragged: the last tile is not full
+    };
+    [[maybe_unused]] int conv_iyr = 0, conv_ixs = 0;
+    [[maybe_unused]] bool conv_kvalid = false;
+    auto conv_tap = [&]() {
+        if constexpr (OP == 1 && !CW) { conv_iyr = cr * a.cdil; conv_ixs = cs * a.cdil_w; conv_kvalid = cr < a.KH; }
+    };
+    auto issue_loads = [&](auto ragc, int stage, auto firstc, auto countc) {
+        constexpr bool RAG = decltype(ragc)::value;
+        constexpr int FIRST = decltype(firstc)::value, COUNT = decltype(countc)::value;
         char* sbase = lds + stage * STAGE_BYTES;
-        if constexpr (PF > 0) {
-            // the touched dwords are dropped into a scratch corner of LDS: no register is tied up and
-            // the loads are counted by vmcnt like the tile fetches that follow them
-            const uint32_t pk = (uint32_t)(issue_kt + PF) * BKB;
-            const bool pf_live = pk < Kb;
-            auto* scratch = (__attribute__((address_space(3))) void*)(lds + NS * STAGE_BYTES + wave * 256);
-            const uint32_t v = pf_live ? pf_off[0] + pk : OOB;
-            if (pf_isb) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, scratch, 4, (int)v, 0, 0, 0);
-            else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, scratch, 4, (int)v, 0, 0, 0);
+        [[maybe_unused]] uint32_t koff_rag = koff_cur;
+        // the masks of the ragged form are computed inside its (rarely taken) branch, not hoisted in front of it
+        if constexpr (RAG) asm volatile("" : "+v"(koff_rag));
+#pragma unroll
+        for (int q = FIRST; q < FIRST + COUNT; ++q) {
+            if (q < A_LPW) {
+                const int i = q;
+                if constexpr (OP == 0) {
+                    uint32_t v = voffA[i];
+                    if constexpr (RAG) {
+                        const int row = (i * NW + wave) * RPI + lrow;
+                        if (koff_rag + (uint32_t)((lpos ^ swz_of_row(row)) * 16) >= Kb) v = OOB;
+                    }
+                    load_chunk_to_lds(rA_cur, sbase + (i * NW + wave) * 1024, v, ks_cur);
+                } else if constexpr (!CW) {
+                    const int iy = iy0[i] + conv_iyr, ix = ix0[i] + conv_ixs;
+                    const bool ok = conv_kvalid && (unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W;
+                    const uint32_t v = ok ? voffA[i] + (uint32_t)((iy * a.W + ix) * a.CI + cc) * ES : OOB;
+                    load_chunk_to_lds(rA_cur, sbase + (i * NW + wave) * 1024, v, 0u);
+                }
+            } else {
+                const int i = q - A_LPW;
+                uint32_t v = voffB[i];
+                if constexpr (RAG) {
+                    const int row = (i * NW + wave) * RPI + lrow;
+                    if (koff_rag + (uint32_t)((lpos ^ swz_of_row(row)) * 16) >= Kb) v = OOB;
+                }
+                load_chunk_to_lds(rB_cur, sbase + A_BYTES + (i * NW + wave) * 1024, v, ks_cur);
+            }
         }
-        tile_offsets();
-#pragma unroll
-        for (int i = 0; i < A_LPW; ++i) load_chunk_to_lds(rsrcA, sbase + (i * NW + wave) * 1024, offA[i]);
-#pragma unroll
-        for (int i = 0; i < B_LPW; ++i) load_chunk_to_lds(rsrcB, sbase + A_BYTES + (i * NW + wave) * 1024, offB[i]);
+    };
+    auto end_issue = [&]() {
+        if constexpr (OP == 1 && !CW) {
+            // advance the lane's (kh, kw, ci) position by one k-tile
+            cc += BKB / ES;
+            while (cc >= a.CI) { cc -= a.CI; if (++cs == a.KW) { cs = 0; ++cr; } }
+        }
         advance_issue();
     };
-
-    // path 1: fetch k-tile `issue_kt` into register set SET; later copy a set into an LDS stage
-    v4i regA[LOADM ? 2 : 1][LOADM ? (A_LPW > 0 ? A_LPW : 1) : 1], regB[LOADM ? 2 : 1][LOADM ? B_LPW : 1];
-    auto issue_regs = [&](auto setc) {
-        constexpr int SET = decltype(setc)::value;
-        tile_offsets();
-#pragma unroll
-        for (int i = 0; i < A_LPW; ++i) regA[SET][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (int)offA[i], 0, 0);
-#pragma unroll
-        for (int i = 0; i < B_LPW; ++i) regB[SET][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrcB, (int)offB[i], 0, 0);
-        ++issue_kt;
-    };
-    auto write_lds = [&](auto setc, int stage) {
-        constexpr int SET = decltype(setc)::value;
-        char* sbase = lds + stage * STAGE_BYTES + lane * 16;
-#pragma unroll
-        for (int i = 0; i < A_LPW; ++i) *(v4i*)(sbase + (i * NW + wave) * 1024) = regA[SET][i];
-#pragma unroll
-        for (int i = 0; i < B_LPW; ++i) *(v4i*)(sbase + A_BYTES + (i * NW + wave) * 1024) = regB[SET][i];
+    using TrueC = std::integral_constant<bool, true>;
+    using FalseC = std::integral_constant<bool, false>;
+    auto issue_tile = [&](int stage) {          // the whole tile at once (prologue)
+        const bool rag = begin_issue();
+        conv_tap();
+        if (rag) issue_loads(TrueC{}, stage, std::integral_constant<int, 0>{}, std::integral_constant<int, LPT>{});
+        else issue_loads(FalseC{}, stage, std::integral_constant<int, 0>{}, std::integral_constant<int, LPT>{});
+        end_issue();
     };
 
     // ---- per-lane MFMA operand addresses ----
     const int lr = lane % MT, lq = lane / MT;
 
     // ---- conv window mode: the window itself (dynamic LDS) and the per-row tap masks ----
-    extern __shared__ __attribute__((aligned(1024))) char win[];
     const int w_pitch = a.CI * ES;                       // bytes of one pixel (all channels)
     const int w_cch = CW ? w_pitch / BKB : 1;            // k-tiles per tap
     uint32_t tapmask[CW ? TM : 1];                       // bit t: tap t of this lane's pixel i is inside the image
     if constexpr (CW) {
+        const rsrc_t rA = make_rsrc(baseA, a_bytes);
         const int w_rows = BM + 2 * (a.cpad * a.W + a.cpad_w);  // pixels the BM outputs can reach
         const int cpp = w_pitch / 16;                    // 16-byte chunks per pixel
         const int n_instr = (w_rows * cpp + 63) / 64;    // 1 KiB wave loads that cover the window
@@ -445,8 +431,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
             const int src = (pos & ~(CPR - 1)) | ((pos & (CPR - 1)) ^ swz_of_row(wrow));
             const int gp = gp0 + wrow;
             const uint32_t v = (wrow < w_rows && gp >= 0) ? (uint32_t)gp * (uint32_t)w_pitch + src * 16 : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (__attribute__((address_space(3))) void*)(win + q * 1024),
-                                                     16, (int)v, 0, 0, 0);
+            load_chunk_to_lds(rA, win + q * 1024, v, 0u);
         }
         // masks: pixel of fragment row i by one division, the following rows (MT further each) by carry
         const int hw = a.H * a.W;
@@ -490,25 +475,29 @@ hrn_mfma_kernel(const HrnKArgs a) {
     };
     clear_acc();
 
+    // Operand fragments, double-buffered in registers.  Read slot r of a step: r < TN is B fragment r, the others are
+    // the A fragments in row-tile order - the order in which the MFMAs of the step consume them (the first row of
+    // MFMAs needs every B fragment).
     v4i fa[2][TM], fb[2][TN];
-    auto read_frags = [&](int buf, int stage_off, int kk) {
-        const int ko = g16 ^ (kk * KSB);
-        if constexpr (CW) {
-            const int tapoff = (rd_r < a.KH) ? rd_r * a.W + rd_s : 0;    // r*W + s pixels; 0 past the last tap
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
+    constexpr int NRD = TM + TN;
+    auto read_slot = [&](int buf, int stage_off, int kk, int r) {
+        if (r < TN) {
+            fb[buf][r] = *(const v4i*)(lds + stage_off + b_lane + r * MT * BKB + (g16 ^ (kk * KSB)));
+        } else {
+            const int i = r - TN;
+            if constexpr (CW) {
+                const int tapoff = (rd_r < a.KH) ? rd_r * a.W + rd_s : 0;    // r*W + s pixels; 0 past the last tap
                 const int wrow = w_lane + i * MT + tapoff;
                 const int kc = (kk * CPS + lq) ^ swz_of_row(wrow);
                 fa[buf][i] = *(const v4i*)(win + wrow * w_pitch + rd_cch * BKB + kc * 16);
+            } else {
+                fa[buf][i] = *(const v4i*)(lds + stage_off + a_lane + i * MT * BKB + (g16 ^ (kk * KSB)));
             }
-        } else {
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                fa[buf][i] = *(const v4i*)(lds + stage_off + a_lane + i * MT * BKB + ko);
         }
+    };
+    auto read_frags = [&](int buf, int stage_off, int kk) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-            fb[buf][j] = *(const v4i*)(lds + stage_off + b_lane + j * MT * BKB + ko);
+        for (int r = 0; r < NRD; ++r) read_slot(buf, stage_off, kk, r);
     };
     // window mode: move the reader to the next k-tile (channel chunks inside a tap first, then kw, then kh)
     auto advance_reader = [&]() {
@@ -517,36 +506,39 @@ hrn_mfma_kernel(const HrnKArgs a) {
         }
     };
     int mm_tap = 0, mm_cch = 0;                           // window mode: tap of the k-tile being MULTIPLIED
-    v4i amask[CW ? TM : 1];
+    uint32_t tap_bit = 0;
     auto set_masks = [&]() {
         if constexpr (CW) {
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int on = -(int)((tapmask[i] >> mm_tap) & 1u);
-                amask[i] = (v4i){on, on, on, on};
-            }
+            tap_bit = mm_tap;
             if (++mm_cch == w_cch) { mm_cch = 0; ++mm_tap; }
         }
     };
-    auto mfma_step = [&](int buf) {
-        if constexpr (DT == 1) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                int s = bsum[j];
-                s = __builtin_amdgcn_sdot4(fb[buf][j].x, 0x01010101, s, false);
-                s = __builtin_amdgcn_sdot4(fb[buf][j].y, 0x01010101, s, false);
-                s = __builtin_amdgcn_sdot4(fb[buf][j].z, 0x01010101, s, false);
-                s = __builtin_amdgcn_sdot4(fb[buf][j].w, 0x01010101, s, false);
-                bsum[j] = s;
-            }
+    // the A fragment of row-tile i as the MFMA takes it: window taps in the padding contribute zero, uint8 becomes
+    // int8 by subtracting 128 (the sign-bit flip; the epilogue adds 128 * sum_k B back)
+    auto a_operand = [&](int buf, int i) {
+        v4i av = fa[buf][i];
+        if constexpr (CW) {
+            const int on = -(int)((tapmask[i] >> tap_bit) & 1u);
+            av = av & (v4i){on, on, on, on};
         }
+        if constexpr (DT == 1) av = av ^ (int)0x80808080;
+        return av;
+    };
+    // uint8 path: sum_k B[n,k] of the step's B fragments.  The WM waves of one column hold the same fragments, so
+    // they take turns: wave row w sums the steps with step % WM == w, the epilogue adds the WM partial sums.
+    auto bsum_step = [&](int buf, int step) {
+        if constexpr (DT == 1) {
+            if (WM == 1 || (step & (WM - 1)) == wm_idx) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            v4i av = fa[buf][i];
-            if constexpr (CW) av = av & amask[i];               // taps in the padding contribute zero
-            if constexpr (DT == 1) av = av ^ (int)0x80808080;   // u8 -> s8 by subtracting 128
-#pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = mfma(fb[buf][j], av, acc[i][j]);
+                for (int j = 0; j < TN; ++j) {
+                    int s = bsum[j];
+                    s = __builtin_amdgcn_sdot4(fb[buf][j].x, 0x01010101, s, false);
+                    s = __builtin_amdgcn_sdot4(fb[buf][j].y, 0x01010101, s, false);
+                    s = __builtin_amdgcn_sdot4(fb[buf][j].z, 0x01010101, s, false);
+                    s = __builtin_amdgcn_sdot4(fb[buf][j].w, 0x01010101, s, false);
+                    bsum[j] = s;
+                }
+            }
         }
     };
 
@@ -554,7 +546,8 @@ hrn_mfma_kernel(const HrnKArgs a) {
     // MFMA was issued as (B fragment, A fragment), so a lane holds 4 consecutive n for one m:
     //   m = lr, n = (r/4)*8 + lq*4 + r%4   (32x32)     m = lr, n = lq*4 + r   (16x16)
     auto store_tile = [&]() {
-        int* bs_lds = (int*)(lds + EPI_OFF);
+        char* const epi = CW ? win : lds + EPI_OFF;
+        int* bs_lds = (int*)epi;
         if constexpr (DT == 1) {
             // 128 * sum_k B[n,k] completes the u8 x s8 product computed as (u8-128) x s8
             if constexpr (PERS) wait_and_barrier<63, 0>();     // the stages stay live: LDS traffic only, no drain
@@ -564,65 +557,82 @@ hrn_mfma_kernel(const HrnKArgs a) {
                 int s = bsum[j];
 #pragma unroll
                 for (int d = MT; d < 64; d <<= 1) s += __shfl_xor(s, d, 64);
-                if (wm_idx == 0 && lq == 0) bs_lds[wn_idx * WTN + j * MT + lr] = s;
+                if (lq == 0) bs_lds[wm_idx * BN + wn_idx * WTN + j * MT + lr] = s;
             }
             if constexpr (PERS) wait_and_barrier<63, 0>();
             else __syncthreads();
         }
+        // column sums of the 4 consecutive outputs a lane holds, all wave rows added
+        auto colsum4 = [&](int nl) {
+            v4i bs = *(const v4i*)(bs_lds + nl);
+#pragma unroll
+            for (int w = 1; w < WM; ++w) bs += *(const v4i*)(bs_lds + w * BN + nl);
+            return bs;
+        };
 
-        char* Cb = (char*)a.C + (int64_t)c_bz * a.sC * OES;
-        const bool do_store = !(ABL & 16) || a.K == 0x7fffffff;   // the ablation keeps the stores reachable but never takes them
-        if constexpr (EPI == 1) {
-            // LDS-staged epilogue: a wave parks one MFMA row-tile (MT rows x WTN columns) of its result in a private,
+        char* Cb = (char*)a.C + ((int64_t)slice * a.batch + c_bz) * a.sC * OES;
+        const bool do_store = !(ABL & 16) || a.K == 0x7fffffff;   // the study switch keeps the stores reachable but never takes them
+        if constexpr (EPI >= 1) {
+            // LDS-staged epilogue: a wave parks one MFMA row-tile (MT rows x SW columns) of its result in a private,
             // padded LDS strip, then streams it out with 16 bytes per lane, whole row segments per store instruction.
             if constexpr (DT == 0 && !PERS) wait_and_barrier<0, 0>();   // (the int8 path has synchronised above) stages are dead now
             [[maybe_unused]] const rsrc_t rsrcC = make_rsrc(Cb, (uint32_t)a.M * (uint32_t)a.ldc * OES);
-            char* strip = lds + EPI_OFF + EPI_BASE + wave * (MT * EPI_PITCH);
-            constexpr int CPRW = WTN * OES / 16;               // 16-byte chunks per strip row
+            char* strip = epi + EPI_BASE + wave * (MT * EPI_PITCH);
+            constexpr int CPRW = SW * OES / 16;                // 16-byte chunks per strip row
             constexpr int EPC = 16 / OES;                      // output elements per chunk
+            constexpr int TNS = TN / ESPLIT;                   // MFMA column tiles per strip
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j) {
+                for (int h = 0; h < ESPLIT; ++h) {
 #pragma unroll
-                    for (int g = 0; g < ACC_N / 4; ++g) {
-                        const int cl = j * MT + g * 8 + lq * 4;          // column inside the wave tile
-                        char* dst = strip + lr * EPI_PITCH + cl * OES;
-                        if constexpr (DT == 0) {
-                            v4h o;
+                    for (int js = 0; js < TNS; ++js) {
+                        const int j = h * TNS + js;
 #pragma unroll
-                            for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[i][j][g * 4 + r];
-                            *(v4h*)dst = o;
+                        for (int g = 0; g < ACC_N / 4; ++g) {
+                            const int cl = js * MT + g * 8 + lq * 4;         // column inside the strip
+                            char* dst = strip + lr * EPI_PITCH + cl * OES;
+                            if constexpr (DT == 0 && !SPLITK) {
+                                v4h o;
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[i][j][g * 4 + r];
+                                *(v4h*)dst = o;
+                            } else if constexpr (DT == 0) {
+                                v4f o;
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r];
+                                *(v4f*)dst = o;
+                            } else {
+                                const v4i bs = colsum4(wn_idx * WTN + h * SW + cl);
+                                v4i o;
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r] + 128 * bs[r];
+                                *(v4i*)dst = o;
+                            }
+                        }
+                    }
+                    asm volatile("" ::: "memory");     // LDS serves one wave's requests in order: the reads below see the writes
+#pragma unroll
+                    for (int it = 0; it < MT * CPRW / 64; ++it) {
+                        const int c = it * 64 + lane;
+                        const int row = c / CPRW, cc2 = c % CPRW;
+                        const v4i val = *(const v4i*)(strip + row * EPI_PITCH + cc2 * 16);
+                        const int m = m0 + wm_idx * WTM + i * MT + row;
+                        const int n = n0 + wn_idx * WTN + h * SW + cc2 * EPC;
+                        if constexpr (PERS) {
+                            // always issued, so that every wave has exactly STORES_PER_TILE stores per tile in flight
+                            const uint32_t off = (m < a.M && n + EPC <= a.N) ? (uint32_t)(m * a.ldc + n) * OES : OOB;
+                            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(unsigned int __attribute__((ext_vector_type(4))), val), rsrcC, (int)off, 0, 0);
                         } else {
-                            const v4i bs = *(const v4i*)(bs_lds + wn_idx * WTN + cl);
-                            v4i o;
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r] + 128 * bs[r];
-                            *(v4i*)dst = o;
+                            char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
+                            if (do_store && m < a.M) {
+                                if (n + EPC <= a.N) *(v4i*)dst = val;
+                                else if (OES == 2 && n + 4 <= a.N) *(long*)dst = ((long)(uint32_t)val.y << 32) | (uint32_t)val.x;
+                            }
                         }
                     }
+                    asm volatile("" ::: "memory");
                 }
-                asm volatile("" ::: "memory");     // LDS serves one wave's requests in order: the reads below see the writes
-#pragma unroll
-                for (int it = 0; it < MT * CPRW / 64; ++it) {
-                    const int c = it * 64 + lane;
-                    const int row = c / CPRW, cc2 = c % CPRW;
-                    const v4i val = *(const v4i*)(strip + row * EPI_PITCH + cc2 * 16);
-                    const int m = m0 + wm_idx * WTM + i * MT + row;
-                    const int n = n0 + wn_idx * WTN + cc2 * EPC;
-                    if constexpr (PERS) {
-                        // always issued, so that every wave has exactly STORES_PER_TILE stores per tile in flight
-                        const uint32_t off = (m < a.M && n + EPC <= a.N) ? (uint32_t)(m * a.ldc + n) * OES : OOB;
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(unsigned int __attribute__((ext_vector_type(4))), val), rsrcC, (int)off, 0, 0);
-                    } else {
-                        char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
-                        if (do_store && m < a.M) {
-                            if (n + EPC <= a.N) *(v4i*)dst = val;
-                            else if (DT == 0 && n + 4 <= a.N) *(long*)dst = ((long)(uint32_t)val.y << 32) | (uint32_t)val.x;
-                        }
-                    }
-                }
-                asm volatile("" ::: "memory");
             }
         } else {
 #pragma unroll
@@ -636,13 +646,18 @@ hrn_mfma_kernel(const HrnKArgs a) {
                         const int n = n0 + nl;
                         if (do_store && m < a.M && n < a.N) {
                             char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
-                            if constexpr (DT == 0) {
+                            if constexpr (DT == 0 && !SPLITK) {
                                 v4h o;
 #pragma unroll
                                 for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[i][j][g * 4 + r];
                                 *(v4h*)dst = o;
+                            } else if constexpr (DT == 0) {
+                                v4f o;
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r];
+                                *(v4f*)dst = o;
                             } else {
-                                const v4i bs = *(const v4i*)(bs_lds + nl);
+                                const v4i bs = colsum4(nl);
                                 v4i o;
 #pragma unroll
                                 for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r] + 128 * bs[r];
@@ -655,95 +670,120 @@ hrn_mfma_kernel(const HrnKArgs a) {
         }
     };
 
-    if constexpr (LOADM == 0) {
-        // ---- prologue: fill all stages, wait for tile 0 ----
-    #pragma unroll
-        for (int s = 0; s < NS; ++s) issue_tile(s);
-        wait_and_barrier<(NS - 1) * LPT, 0>();
-        read_frags(0, 0, 0);
-
-        int stage = 0;
-        auto run_tile = [&](const bool stores_between) {
-            for (int kt = 0; kt < KT; ++kt) {
-                const int stage_off = stage * STAGE_BYTES;
-                const int next_stage = (stage + 1 == NS) ? 0 : stage + 1;
-                set_masks();
-    #pragma unroll
-                for (int kk = 0; kk < KS; ++kk) {
-                    const int cur = kk & 1;
-                    if (kk == KS - 1) {
-                        // every fragment of tile kt is in registers: publish tile kt+1, recycle this stage
-                        if constexpr (PERS) {
-                            if (stores_between && kt <= NS - 2) wait_and_barrier<(NS - 2) * LPT + STORES_PER_TILE, 0>();
-                            else wait_and_barrier<(NS - 2) * LPT, 0>();
-                        } else if constexpr (ABL & 4) {
-                            wait_only<(NS - 2) * LPT, 0>();
-                        } else {
-                            wait_and_barrier<(NS - 2) * LPT, 0>();
-                        }
-                        if (!(ABL & 2)) issue_tile(stage);
-                        advance_reader();
-                        if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, next_stage * STAGE_BYTES, 0);
-                    } else {
-                        if (!(ABL & 1) || kt == 0) read_frags(cur ^ 1, stage_off, kk + 1);
-                    }
-                    if (!(ABL & 8)) mfma_step(cur);
-                    // pin the issue order: fragment reads (and, in the last step, the tile fetch) are
-                    // spread between the MFMAs of this step instead of being sunk behind them
-                    if (kk == KS - 1) sched_pattern<0, TM + TN, TM * TN, LPT>();
-                    else sched_pattern<0, TM + TN, TM * TN, 0>();
-                }
-                stage = next_stage;
-            }
-            store_tile();
-        };
-        if constexpr (PERS) {
-            for (int ct = blockIdx.x; ct < total; ct += (int)gridDim.x) {
-                tile_coords(ct, c_bz, c_tile_m, c_tile_n, c_tin, c_gsz);
-                m0 = c_tile_m * BM; n0 = c_tile_n * BN;
-                // the stores of the previous tile's epilogue sit between the fetches that were issued before it and
-                // the ones issued after it; while such a fetch is the one waited for, the wait allows for them
-                run_tile(ct != (int)blockIdx.x && KT >= NS - 1);
-                clear_acc();
-            }
-        } else {
-            run_tile(false);
-        }
-    } else {
-        // ---- register-staged pipeline: tile t is requested during tile t-3's last k-step, copied into LDS
-        // during tile t-1 and multiplied as tile t: two tile-times for the data to arrive ----
-        using S0 = std::integral_constant<int, 0>;
-        using S1 = std::integral_constant<int, 1>;
-        issue_regs(S0{});
-        issue_regs(S1{});
-        write_lds(S0{}, 0);
-        wait_and_barrier<63, 0>();
-        issue_regs(S0{});
-        read_frags(0, 0, 0);
-        auto body = [&](auto parity) {
-            constexpr int P = decltype(parity)::value;      // LDS stage of the tile being multiplied
-            using Other = std::integral_constant<int, 1 - P>;
+    // ---- prologue: fill all stages, wait for tile 0 ----
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) {
-                const int cur = kk & 1;
-                if (kk == KS - 2) write_lds(Other{}, 1 - P);       // next tile: registers -> the free LDS stage
-                if (kk == KS - 1) {
-                    wait_and_barrier<63, 0>();                      // LDS writes visible, old stage drained
-                    issue_regs(Other{});                            // request the tile three ahead
-                    read_frags(cur ^ 1, (1 - P) * STAGE_BYTES, 0);
-                } else {
-                    read_frags(cur ^ 1, P * STAGE_BYTES, kk + 1);
-                }
-                if (!(ABL & 8)) mfma_step(cur);
-                if (kk == KS - 1) sched_pattern<0, TM + TN, TM * TN, A_LPW + B_LPW, 0>();
-                else if (kk == KS - 2) sched_pattern<0, TM + TN, TM * TN, 0, A_LPW + B_LPW>();
-                else sched_pattern<0, TM + TN, TM * TN, 0, 0>();
-            }
+    for (int s = 0; s < NS; ++s) issue_tile(s);
+    wait_and_barrier<(NS - 1) * LPT, 0>();
+    read_frags(0, 0, 0);
+
+    int stage = 0;
+    // One k-step: the MFMAs of register buffer `cur`, row-tile by row-tile, with the fragment reads of the next step
+    // (into the other buffer) and - in the last step of a k-tile - the wave loads of the tile that recycles this stage
+    // issued between the rows.  The source order IS the issue order: every row ends in a scheduling fence.  Loads
+    // come first (the next tile's fragment reads may not pass them: both touch LDS), over the first rows of the last
+    // step; reads fill the remaining rows but leave the final row free, so that the barrier of the next tile does
+    // not wait for a read that was just issued.
+    auto kstep = [&](auto lastc, const bool rag, const int cur, const int rd_stage_off, const int rd_kk, const int kt,
+                     const int step) {
+        constexpr bool LAST = decltype(lastc)::value;
+        constexpr int NLD = (LAST && !(ABL & 2)) ? LPT : 0;
+        // rows of the last step that carry the tile's loads: HRN_LSPREAD 0 = none (all loads right behind the barrier),
+        // 1 = the first quarter of the rows, 2 = half, 3 = all but the last two; spreading the requests smooths the
+        // demand on the L2 (every workgroup of an XCD reaches its barrier at about the same time), at the price of a
+        // later arrival of the tile
+        constexpr int LROWS_WANT = LSPREAD == 0 ? 0 : (LSPREAD == 1 ? TM / 4 : (LSPREAD == 2 ? TM / 2 : TM - 2));
+        constexpr int LROWS = NLD == 0 ? 0 : (LROWS_WANT < 0 ? 0 : (LROWS_WANT > TM - 1 ? TM - 1 : (LROWS_WANT == 0 && LSPREAD > 0 && TM >= 2 ? 1 : LROWS_WANT)));
+        constexpr int RROWS_ALL = TM - LROWS;                                         // rows left for the reads
+        constexpr int RROWS = RROWS_ALL >= 2 ? RROWS_ALL - 1 : RROWS_ALL;             // ... minus the free final row
+        const bool do_reads = !(ABL & 1) || kt == 0;
+        // the ragged form differs in the loads only, so the branch (wave-uniform) goes around just these
+        auto loads = [&](auto firstc, auto countc) {
+            if (rag) issue_loads(TrueC{}, stage, firstc, countc);
+            else issue_loads(FalseC{}, stage, firstc, countc);
         };
-        for (int kt = 0; kt < KT; kt += 2) {
-            body(S0{});
-            if (kt + 1 < KT) body(S1{});
+        if constexpr (LROWS == 0 && NLD > 0) loads(std::integral_constant<int, 0>{}, std::integral_constant<int, NLD>{});
+        v4i av = a_operand(cur, 0);
+        auto row = [&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            if constexpr (i < LROWS) {
+                constexpr int f = NLD * i / LROWS, n = NLD * (i + 1) / LROWS - f;
+                loads(std::integral_constant<int, f>{}, std::integral_constant<int, n>{});
+            } else if constexpr (i - LROWS < RROWS) {
+                constexpr int f = NRD * (i - LROWS) / RROWS, n = NRD * (i - LROWS + 1) / RROWS - f;
+                if (do_reads) {
+#pragma unroll
+                    for (int r = f; r < f + n; ++r) read_slot(cur ^ 1, rd_stage_off, rd_kk, r);
+                }
+            }
+            if (!(ABL & 8)) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma(fb[cur][j], av, acc[i][j]);
+            }
+            if constexpr (i + 1 < TM) av = a_operand(cur, i + 1);      // ready before the next row's MFMAs ask for it
+            if constexpr (SCHED == 1) __builtin_amdgcn_sched_barrier(0);
+        };
+        auto rows = [&](auto self, auto ic) -> void {
+            row(ic);
+            if constexpr (decltype(ic)::value + 1 < TM) self(self, std::integral_constant<int, decltype(ic)::value + 1>{});
+        };
+        rows(rows, std::integral_constant<int, 0>{});
+        if constexpr (SCHED == 0) sched_hint<0, TM + TN, TM * TN, NLD>();
+        bsum_step(cur, step);
+    };
+    // One k-tile.  P = register buffer that holds the fragments of its first k-step (the buffers alternate per
+    // k-step, so with an odd number of k-steps per tile P alternates per tile).
+    auto tile_body = [&](auto pc, const int kt, const bool stores_between) {
+        constexpr int P = decltype(pc)::value;
+        const int stage_off = stage * STAGE_BYTES;
+        const int next_stage = (stage + 1 == NS) ? 0 : stage + 1;
+        set_masks();
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            const int cur = (kk + P) & 1;
+            if (kk == KS - 1) {
+                // every fragment of tile kt is in registers: publish tile kt+1, recycle this stage
+                if constexpr (PERS) {
+                    if (stores_between && kt <= NS - 2) wait_and_barrier<(NS - 2) * LPT + STORES_PER_TILE, 0>();
+                    else wait_and_barrier<(NS - 2) * LPT, 0>();
+                } else if constexpr (ABL & 4) {
+                    wait_only<(NS - 2) * LPT, 0>();
+                } else {
+                    wait_and_barrier<(NS - 2) * LPT, 0>();
+                }
+                const bool rag = begin_issue();
+                conv_tap();
+                advance_reader();
+                kstep(TrueC{}, rag, cur, next_stage * STAGE_BYTES, 0, kt, kt * KS + kk);
+                if (!(ABL & 2)) end_issue();
+            } else {
+                kstep(FalseC{}, false, cur, stage_off, kk + 1, kt, kt * KS + kk);
+            }
+        }
+        stage = next_stage;
+    };
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    auto run_tile = [&](const bool stores_between) {
+        if constexpr (KS % 2 == 0) {
+            for (int kt = 0; kt < KT; ++kt) tile_body(P0{}, kt, stores_between);
+        } else {
+            for (int kt = 0; kt < KT; kt += 2) {
+                tile_body(P0{}, kt, stores_between);
+                if (kt + 1 < KT) tile_body(P1{}, kt + 1, stores_between);
+            }
         }
         store_tile();
+    };
+    if constexpr (PERS) {
+        for (int ct = blockIdx.x; ct < total; ct += (int)gridDim.x) {
+            tile_coords(ct, c_bz, c_tile_m, c_tile_n);
+            m0 = c_tile_m * BM; n0 = c_tile_n * BN;
+            // the stores of the previous tile's epilogue sit between the fetches that were issued before it and
+            // the ones issued after it; while such a fetch is the one waited for, the wait allows for them
+            run_tile(ct != (int)blockIdx.x && KT >= NS - 1);
+            clear_acc();
+        }
+    } else {
+        run_tile(false);
     }
 }

@@ -16,8 +16,9 @@ def _chk(t, dtype):
         raise ValueError("expected a contiguous CUDA tensor of %s, got %s %s" % (dtype, t.dtype, t.device))
 
 
-def gemm(mod, A, Bm, out=None, group_m=8):
-    """C = A @ Bm.T for A (M,K), Bm (N,K), or batched (b,M,K) x (b,N,K) -> (b,M,N)."""
+def gemm(mod, A, Bm, out=None, group_m=8, split_k=0):
+    """C = A @ Bm.T for A (M,K), Bm (N,K), or batched (b,M,K) x (b,N,K) -> (b,M,N).  ``split_k`` is the number of
+    K slices for a split-K instance (the module supplies the workspace)."""
     f16 = mod.desc.dtype == B.HRN_DT_F16
     _chk(A, torch.float16 if f16 else torch.uint8)
     _chk(Bm, torch.float16 if f16 else torch.int8)
@@ -29,7 +30,7 @@ def gemm(mod, A, Bm, out=None, group_m=8):
     oshape = (batch, M, N) if A.dim() == 3 else (M, N)
     if out is None:
         out = torch.empty(oshape, dtype=torch.float16 if f16 else torch.int32, device=A.device)
-    p = B.gemm_problem(batch, M, N, K, group_m)
+    p = B.gemm_problem(batch, M, N, K, group_m, split_k)
     mod.launch(p, A.data_ptr(), Bm.data_ptr(), out.data_ptr(), _stream())
     return out
 
@@ -43,7 +44,7 @@ def unpack_filter_blocked(Wb):
     return Wb.permute(0, 4, 1, 2, 3, 5).reshape(OC * cb, KH, KW, ICC * 4).contiguous()
 
 
-def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8):
+def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8, split_k=0):
     """X (N,H,W,CI), Wt KRSC (CO,KH,KW,CI) -> (N,HO,WO,CO): fp16 -> fp16, or uint8 x int8 -> int32."""
     f16 = mod.desc.dtype == B.HRN_DT_F16
     _chk(X, torch.float16 if f16 else torch.uint8)
@@ -52,7 +53,7 @@ def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8):
     CO, KH, KW, CI2 = Wt.shape
     if CI != CI2:
         raise ValueError("channel mismatch")
-    p = B.conv2d_problem(N, H, W, CI, CO, KH, KW, stride, pad, dil, group_m)
+    p = B.conv2d_problem(N, H, W, CI, CO, KH, KW, stride, pad, dil, group_m, split_k)
     (sh, sw), (ph, pw), (dh, dw) = B._pair(stride), B._pair(pad), B._pair(dil)
     ho = (H - ((KH - 1) * dh + 1) + 2 * ph) // sh + 1
     wo = (W - ((KW - 1) * dw + 1) + 2 * pw) // sw + 1

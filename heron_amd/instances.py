@@ -12,8 +12,8 @@ F16, U8 = B.HRN_DT_F16, B.HRN_DT_U8S8
 GEMM, CONV = B.HRN_OP_GEMM, B.HRN_OP_CONV2D
 
 
-def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, pf=0, load=0, win=0, pers=0):
-    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, pf, 0, load, win, pers)
+def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, win=0, pers=0, split=0, sched=1, spread=2):
+    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, win, pers, split, sched, spread)
 
 
 # (bm, bn, bkb, wm, wn, mfma, stages, swizzle): a spread of the template space used by the parity tests
@@ -30,11 +30,11 @@ PARITY_SHAPES = [
 ]
 
 
-# instances that exercise the optional load paths: (tile tuple, l2_prefetch, load_mode)
 # (tile tuple) instances run with the LDS-staged epilogue as well
 EPILOGUE_VARIANTS = [
     (256, 256, 128, 2, 4, 16, 2, 2),
     (256, 256, 128, 4, 2, 32, 2, 2),
+    (256, 256, 128, 4, 2, 16, 2, 2),
     (256, 256, 64, 2, 4, 32, 4, 3),
     (128, 128, 128, 2, 2, 32, 2, 1),
     (64, 64, 128, 4, 2, 16, 3, 1),
@@ -42,29 +42,42 @@ EPILOGUE_VARIANTS = [
     (128, 64, 128, 2, 1, 32, 2, 1),
 ]
 
-PARITY_VARIANTS = [
-    ((256, 256, 128, 4, 2, 32, 2, 2), 1, 0),
-    ((128, 128, 128, 2, 2, 32, 3, 1), 2, 0),
-    ((256, 256, 128, 4, 2, 32, 2, 2), 0, 1),
-    ((128, 64, 128, 2, 1, 16, 2, 1), 0, 1),
+# one MFMA k-step per k-tile (64-byte rows with 16x16 MFMAs): the register buffers alternate per tile
+SINGLE_STEP_VARIANTS = [
+    (256, 256, 64, 2, 4, 16, 5, 3),
+    (256, 256, 64, 4, 2, 16, 4, 3),
+    (128, 128, 64, 2, 2, 16, 3, 3),
+    (64, 64, 64, 1, 2, 16, 2, 3),
 ]
 
 
 def variant_descs():
     out = []
-    for t, pf, load in PARITY_VARIANTS:
-        out.append(D(F16, GEMM, *t, pf=pf, load=load))
-        out.append(D(U8, GEMM, *t, pf=pf, load=load))
-    out.append(D(F16, CONV, 128, 64, 128, 2, 1, 16, 2, 1, load=1))
-    for t in EPILOGUE_VARIANTS:
+    for t in EPILOGUE_VARIANTS + SINGLE_STEP_VARIANTS:
         out.append(D(F16, GEMM, *t, epi=1))
         out.append(D(U8, GEMM, *t, epi=1))
+    out.append(D(F16, GEMM, 64, 64, 64, 1, 2, 16, 2, 3))
+    out.append(D(U8, GEMM, 128, 128, 64, 4, 1, 16, 3, 3))
     out.append(D(F16, CONV, 256, 64, 128, 8, 1, 16, 2, 1, epi=1))
     out.append(D(F16, CONV, 256, 64, 128, 8, 1, 16, 2, 1, epi=1, win=1))
     out.append(D(F16, CONV, 128, 64, 128, 2, 2, 32, 3, 1, win=1))
     out.append(D(F16, CONV, 64, 64, 64, 2, 2, 32, 2, 2, epi=1, win=1))
     out.append(D(F16, CONV, 128, 64, 128, 2, 1, 32, 2, 1, epi=1))
+    out.append(D(F16, CONV, 128, 64, 64, 4, 1, 16, 3, 3, epi=1))
+    out.append(D(F16, CONV, 128, 64, 128, 4, 1, 16, 2, 2, epi=1, win=1))
     return out
+
+
+def splitk_descs():
+    """Split-K instances of the parity suite (GEMM and im2col conv, both element kinds, both epilogues)."""
+    return [
+        D(F16, GEMM, 64, 64, 128, 2, 2, 16, 3, 1, epi=1, split=1),
+        D(F16, GEMM, 128, 64, 64, 2, 2, 32, 3, 2, epi=0, split=1),
+        D(U8, GEMM, 64, 64, 128, 2, 2, 16, 3, 1, epi=1, split=1),
+        D(U8, GEMM, 64, 128, 128, 1, 2, 32, 2, 1, epi=0, split=1),
+        D(F16, CONV, 64, 64, 128, 2, 2, 16, 3, 1, epi=1, split=1),
+        D(U8, CONV, 64, 64, 64, 2, 2, 32, 2, 1, epi=1, split=1),
+    ]
 
 
 def parity_descs():
@@ -113,26 +126,18 @@ def persistent_twin_descs():
     return [D(d.dtype, d.op, *d.as_tuple()[2:10], epi=1) for d in persistent_descs() if d.op == GEMM]
 
 
-# best known instances per benchmark workload (from CGA tuning runs on MI355X and sweeps around their results); the raster group of
-# each is in BEST_GROUP_M
+# small general-purpose instances (smoke, error-path and operator tests); the tuned instances of the benchmark
+# configurations come from the records under tests/quick_start/rocm/tuned/ (heron_amd.tuned)
 BEST = {
-    "gemm_f16": D(F16, GEMM, 256, 256, 128, 2, 4, 16, 2, 2, epi=1),
-    "gemm_f16_4096": D(F16, GEMM, 256, 256, 128, 2, 4, 16, 2, 2, epi=1),
-    "gemm_u8s8": D(U8, GEMM, 256, 256, 128, 2, 4, 16, 2, 2, epi=1),
-    "bmm_f16_qk": D(F16, GEMM, 256, 128, 128, 4, 2, 16, 2, 2, epi=1, pers=1),
-    "bmm_f16_pv": D(F16, GEMM, 64, 64, 128, 4, 2, 16, 3, 1, epi=1, wpe=1),
-    "conv2d_f16": D(F16, CONV, 512, 64, 128, 8, 1, 32, 2, 2, epi=1, win=1),
-    "conv2d_u8s8": D(U8, CONV, 256, 64, 64, 4, 1, 32, 2, 2, epi=1, wpe=2, win=1),
     "small": D(U8, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
     "small_f16": D(F16, GEMM, 64, 64, 128, 1, 1, 32, 3, 1),
 }
 
-BEST_GROUP_M = {"gemm_f16": 4, "gemm_f16_4096": 4, "gemm_u8s8": 4, "bmm_f16_qk": 8, "bmm_f16_pv": 2, "conv2d_f16": 16, "conv2d_u8s8": 32}
-
 
 def all_shipped():
     seen, out = set(), []
-    for d in parity_descs() + variant_descs() + int8_conv_descs() + persistent_descs() + persistent_twin_descs() + list(BEST.values()):
+    for d in (parity_descs() + variant_descs() + int8_conv_descs() + persistent_descs() + persistent_twin_descs() + splitk_descs()
+              + list(BEST.values())):
         if d.as_tuple() not in seen:
             seen.add(d.as_tuple())
             out.append(d)

@@ -1,9 +1,12 @@
-"""Boosted-tree cost model on raw knob-value vectors.
+"""Boosted-tree cost model on the feature vectors of measured samples (``Sample.features()``: the task's compact
+features, or the raw knob-value vector when the operator set defines none).
 
 Interface of the reference's XGBoostCostModel (model/xgboost_cost_model.py:66-104): ``train(perf_buffer)``,
-``fit(x, y)``, ``predict(samples)`` (ones while untrained) and ``.bst`` (None until trained; exposes
+``fit(x, y)``, ``predict(samples)`` and ``.bst`` (None until trained; exposes
 ``get_score`` for feature ranking).  xgboost is used when importable with the reference's
-parameters (reg, depth 7, eta 0.3); otherwise scikit-learn's gradient boosting stands in.
+parameters (reg, depth 7, eta 0.3); otherwise scikit-learn's gradient boosting stands in.  While untrained the
+reference predicts ones; here the analytic estimate of the feature vector (its last entry, ln(1/seconds)) ranks the
+candidates when the task provides one, so that the first measured batch is not a blind draw.
 """
 import numpy as np
 
@@ -45,6 +48,11 @@ class _XgbBooster:  # pragma: no cover - only with xgboost installed
         return self.bst.get_score(importance_type=importance_type)
 
 
+def feature_matrix(samples):
+    """Rows = what each sample shows the model: its compact features, or its raw point."""
+    return np.array([s.features() if hasattr(s, "features") else s.point for s in samples], dtype=np.float64)
+
+
 class XGBoostCostModel:
     def __init__(self, task, config, num_threads=None, log_interval=25):
         self.task = task
@@ -56,21 +64,33 @@ class XGBoostCostModel:
         self.log_interval = log_interval
         self.bst = None
         self._sample_size = 0
+        # an analytic time estimate ranks candidates before the first measurement (tasks of the MFMA template have one)
+        self.has_prior = getattr(getattr(task, "config", None), "codegen_type", None) == "GPU_MFMA"
 
     def train(self, perf_buffer):
         self.fit(np.array(perf_buffer.data_x), np.array(perf_buffer.data_y))
 
     def fit(self, x_train, y_train, plan_size=30):
-        y_train = y_train / (max(y_train) + 1e-8)
+        x_train = np.asarray(x_train, dtype=np.float64)
+        y_train = np.asarray(y_train, dtype=np.float64)
+        if self.has_prior:
+            # learn the correction to the analytic estimate (last feature, same unit as perf: ln(1/seconds))
+            y_train = y_train - x_train[:, -1]
+        else:
+            y_train = y_train / (max(y_train) + 1e-8)
         index = np.random.permutation(len(x_train))
-        x, y = x_train[index].astype(np.float64), y_train[index]
+        x, y = x_train[index], y_train[index]
         self._sample_size = len(x_train)
         self.bst = _XgbBooster(x, y) if xgb is not None else _SklearnBooster(x, y)
 
     def predict(self, samples, output_margin=False):
-        feas = np.array([s.point for s in samples], dtype=np.float64)
-        if self.bst is None:
-            return np.ones(len(samples))
         if len(samples) == 0:
             return np.zeros(0)
-        return self.bst.predict(feas)
+        if self.bst is None:
+            prior = [s.prior() if hasattr(s, "prior") else None for s in samples]
+            if any(p is None for p in prior):
+                return np.ones(len(samples))
+            prior = np.array(prior, dtype=np.float64)
+            return prior
+        feas = feature_matrix(samples)
+        return (feas[:, -1] if self.has_prior else 0.0) + self.bst.predict(feas)

@@ -1,16 +1,43 @@
-"""Fork-per-chunk parallel sampling with a timeout (multi.py:10-49 of the reference).
+"""Runs a function in a forked child with a time limit (the job abstraction of the reference's multi.py:10-49).
 
-A ``Job`` forks a child that runs ``func(*inputs)`` and sends the result through a queue; ``get``
-waits ``timeout`` seconds, returns 0 on failure and kills the child's whole process tree.
-Children must never call into the HIP library (it is not fork-safe once initialised); sampling
-only touches the constraint solver.
+``Job(func, args, timeout)``: ``start(args)`` forks, ``get()`` returns the child's result, or 0 when the child
+raised, died or outlived ``timeout`` seconds - in which case the child and everything it started are killed.
+Forking copies the parent's task and constraint solver for free, which is why sampling uses it; the children must
+never call into the HIP library (not fork-safe once initialised) - they only run the solver.
 """
-import multiprocessing as _multi
+import multiprocessing
 import signal
+import traceback
 
 import psutil
 
-multi = _multi.get_context("fork")
+_ctx = multiprocessing.get_context("fork")
+multi = _ctx        # kept: callers that want the same start method
+
+
+def _child(func, conn, args):
+    try:
+        out = func(*args)
+    except Exception:  # noqa: BLE001 - the parent gets "no result" at once instead of waiting for the limit
+        traceback.print_exc()
+        out = 0
+    try:
+        conn.send(out)
+    finally:
+        conn.close()
+
+
+def kill_child_processes(parent_pid, sig=signal.SIGTERM):
+    """Signals every descendant of ``parent_pid``."""
+    try:
+        descendants = psutil.Process(parent_pid).children(recursive=True)
+    except psutil.NoSuchProcess:
+        return
+    for proc in descendants:
+        try:
+            proc.send_signal(sig)
+        except psutil.NoSuchProcess:
+            pass
 
 
 class Job:
@@ -18,45 +45,26 @@ class Job:
         self.func = func
         self.attach_info = attach_info
         self.timeout = timeout
+        self._proc = None
+        self._conn = None
 
     def start(self, inputs):
-        self.queue = multi.Queue(2)
-        self.process = multi.Process(target=exec, args=(self.func, self.queue, inputs,))
-        self.process.start()
+        self._conn, child_end = _ctx.Pipe(duplex=False)
+        self._proc = _ctx.Process(target=_child, args=(self.func, child_end, inputs))
+        self._proc.start()
+        child_end.close()
 
     def get(self):
+        result = 0
         try:
-            res = self.queue.get(block=True, timeout=self.timeout)
-        except Exception:  # noqa: BLE001 - timeout or a broken pipe both mean "no result"
-            res = 0
-        if self.process.is_alive():
-            kill_child_processes(self.process.pid)
-            self.process.terminate()
-        self.process.join()
-        self.queue.close()
-        self.queue.join_thread()
-        del self.process
-        del self.queue
-        return res
-
-
-def exec(func, queue, args):
-    try:
-        res = func(*args)
-    except Exception:  # noqa: BLE001 - report the failure at once instead of letting the parent wait for the timeout
-        import traceback
-        traceback.print_exc()
-        res = 0
-    queue.put(res)
-
-
-def kill_child_processes(parent_pid, sig=signal.SIGTERM):
-    try:
-        parent = psutil.Process(parent_pid)
-    except psutil.NoSuchProcess:
-        return
-    for process in parent.children(recursive=True):
-        try:
-            process.send_signal(sig)
-        except psutil.NoSuchProcess:
-            return
+            if self._conn.poll(self.timeout):
+                result = self._conn.recv()
+        except (EOFError, OSError):
+            result = 0                      # the child died before it could answer
+        if self._proc.is_alive():
+            kill_child_processes(self._proc.pid)
+            self._proc.terminate()
+        self._proc.join()
+        self._conn.close()
+        self._proc = self._conn = None
+        return result

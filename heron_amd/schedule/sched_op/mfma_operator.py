@@ -30,8 +30,9 @@ class TemplateSchedule:
         dtype = B.HRN_DT_F16 if self.info['kind'] == 'f16' else B.HRN_DT_U8S8
         op = B.HRN_OP_CONV2D if self.info['operator'] == 'conv2d_nhwc' else B.HRN_OP_GEMM
         return B.make_desc(dtype, op, p['bm'], p['bn'], p['bkb'], p['wm'], p['wn'], p['mfma'], p['stages'],
-                           p['swizzle'], p.get('epilogue', 0), p['waves_per_eu'], p.get('l2_prefetch', 0), 0, 0,
-                           p.get('conv_window', 0), p.get('persistent', 0))
+                           p['swizzle'], p.get('epilogue', 0), p['waves_per_eu'],
+                           p.get('conv_window', 0), p.get('persistent', 0), 1 if p.get('split_k', 1) > 1 else 0,
+                           p.get('sched', 1), p.get('load_spread', 2))
 
     def to_problem(self):
         from ... import backend as B
@@ -40,8 +41,8 @@ class TemplateSchedule:
             c = self.info['conv']
             return B.conv2d_problem(c['N'], c['H'], c['W'], c['CI'], c['CO'], c['KH'], c['KW'],
                                     (c['stride'], c['stride_w']), (c['pad'], c['pad_w']), (c['dil'], c['dil_w']),
-                                    self.params['group_m'])
-        return B.gemm_problem(g['batch'], g['M'], g['N'], g['K'], self.params['group_m'])
+                                    self.params['group_m'], self.params.get('split_k', 1))
+        return B.gemm_problem(g['batch'], g['M'], g['N'], g['K'], self.params['group_m'], self.params.get('split_k', 1))
 
     def describe(self):
         return ", ".join("%s=%s" % kv for kv in sorted(self.params.items()))
@@ -171,7 +172,7 @@ class tileBlockOp(schedOp):
 
 
 class tileKOp(schedOp):
-    """K tiling: bkb bytes of K per LDS row, an even number >= 2 of MFMA k-steps per tile, and k_tiles =
+    """K tiling: bkb bytes of K per LDS row = 1, 2, 4 or 8 MFMA k-steps per tile, and k_tiles =
     ceil(K_bytes / bkb) (the split constraint of the reduce axis, sched_common.py generalTileOp, in covering form:
     the part of the last tile past the end of K is fetched as zeros)."""
 
@@ -179,8 +180,8 @@ class tileKOp(schedOp):
         km = ctx.knob_manager
         kbytes = km.axis_ori_lenth[self.L(stage_name, 'k')]
         bkb = self.knob(ctx, stage_name, 'block_k_bytes', [64, 128, 256], 128)
-        ks = self.var(ctx, stage_name, 'k_steps', 2, 8, 4)
-        km.addCandidates(ks, [2, 4, 8])
+        ks = self.var(ctx, stage_name, 'k_steps', 1, 8, 4)
+        km.addCandidates(ks, [1, 2, 4, 8])
         km.addProd([ks, self.V(stage_name, 'mfma_k_bytes')], bkb)
         kt = self.var(ctx, stage_name, 'k_tiles', 1, kbytes // 64, kbytes // 64)
         kcover = self.var(ctx, stage_name, 'k_cover', kbytes, kbytes + 255, kbytes)
@@ -276,34 +277,10 @@ class ldsStageOp(schedOp):
             km.mems.append(lds)
         ahead = self.var(ctx, stage_name, 'stages_ahead', 1, 4, 1)
         km.addSUM(stages, [ahead, 1])
-        # optional L2 prefetch: one more vector-memory op per lane and tile, at least two waves, GEMM addressing only
-        pf_cands = [0, 1, 2] if s.info['operator'] == 'gemm' else [0]
-        pf = self.knob(ctx, stage_name, 'l2_prefetch', pf_cands, 0)
-        vm_ops = self.var(ctx, stage_name, 'vmem_ops_per_tile', 2, 65, 2)
-        if len(pf_cands) > 1:
-            km.addCandidates(pf, pf_cands)
-            pf_on = self.var(ctx, stage_name, 'l2_prefetch_on', 0, 1, 0)
-            km.addSUM(1, [pf_on, pf.replace("P#", "O#") + '_cand0'])
-            km.addSUM(vm_ops, [self.V(stage_name, 'loads_per_tile'), pf_on])
-            wm1 = self.var(ctx, stage_name, 'waves_minus_1', 0, 15, 0)
-            km.addSUM(self.V(stage_name, 'waves'), [wm1, 1])
-            cap = self.var(ctx, stage_name, 'l2_prefetch_cap', 0, 30, 0)
-            km.addProd([2, wm1], cap)
-            km.addLE(pf, cap)
-            # the touched dwords land in 256 B of LDS per wave, on top of the stages
-            sw = self.var(ctx, stage_name, 'l2_prefetch_scratch_all', 256, 4096, 256)
-            km.addProd([256, self.V(stage_name, 'waves')], sw)
-            scr = self.var(ctx, stage_name, 'l2_prefetch_scratch', 0, 4096, 0)
-            km.addProd([pf_on, sw], scr)
-            total = self.var(ctx, stage_name, 'lds_bytes_total', 4096, lds_limit, 4096)
-            km.addSUM(total, [lds, scr])
-        else:
-            km.addEQ(vm_ops, self.V(stage_name, 'loads_per_tile'))
         inflight = self.var(ctx, stage_name, 'loads_in_flight', 1, ctx.getLimit('max_loads_in_flight'), 1)
-        km.addProd([ahead, vm_ops], inflight)
+        km.addProd([ahead, self.V(stage_name, 'loads_per_tile')], inflight)
         s.params['stages'] = km.get_val(stages)
-        s.params['l2_prefetch'] = km.get_val(pf)
-        ctx.addSchedDesc("LDS stages = %s, L2 prefetch distance = %s\n" % (s.params['stages'], s.params['l2_prefetch']))
+        ctx.addSchedDesc("LDS stages = %s\n" % s.params['stages'])
 
 
 class ldsSwizzleOp(schedOp):
@@ -377,47 +354,102 @@ class registerBudgetOp(schedOp):
         ctx.addSchedDesc("occupancy hint = %s\n" % s.params['waves_per_eu'])
 
 
+class splitKOp(schedOp):
+    """Split-K: the reduction is cut into ``split_k`` slices that run as separate workgroups and a second pass adds
+    their partial sums (for small M*N with long K, where the output tiles alone cannot fill the CUs).  A slice holds
+    at least one k-tile; splitting is only offered while the output tiles number at most one per CU, and it
+    excludes the input window and (in persistentOp) the persistent launch.  The kernel then writes 4-byte partial sums
+    whatever the element type.  The reference never splits the reduce axis over blocks (ops/cuda/dense.py:18-26 binds
+    only spatial axes to blockIdx); its counterpart is the rfactor-free reduce split of generalTileOp."""
+
+    def perform(self, s, stage_name, ctx):
+        km = ctx.knob_manager
+        g = s.info['gemm_view']
+        cus = ctx.getLimit('cu_count')
+        cands = [1, 2, 4, 8, 16]
+        sk = self.knob(ctx, stage_name, 'split_k', cands, 1)
+        km.addCandidates(sk, cands)
+        on = self.var(ctx, stage_name, 'split_k_on', 0, 1, 0)
+        km.addSUM(1, [on, sk.replace("P#", "O#") + '_cand0'])
+        km.addLE(sk, self.V(stage_name, 'k_tiles'))
+        tiles = self.var(ctx, stage_name, 'output_tiles', 1, 1 << 24, 1)
+        km.addProd([self.V(stage_name, 'grid_m'), self.V(stage_name, 'grid_n')], tiles)
+        gated = self.var(ctx, stage_name, 'split_k_output_tiles', 0, max(1, cus // max(1, g['batch'])), 0)
+        km.addProd([on, tiles], gated)
+        sw = self.var(ctx, stage_name, 'split_k_plus_window', 0, 1, 0)
+        km.addSUM(sw, [on, self.P(stage_name, 'conv_window')])
+        # bytes of an output element as the kernel stores it
+        oes = self.var(ctx, stage_name, 'out_elem_bytes', 2, 4, 4)
+        if s.info['kind'] == 'f16':
+            extra = self.var(ctx, stage_name, 'out_elem_bytes_extra', 0, 2, 0)
+            km.addProd([2, on], extra)
+            km.addSUM(oes, [2, extra])
+        else:
+            km.addEQ(oes, 4)
+        s.params['split_k'] = km.get_val(sk)
+        ctx.addSchedDesc("split_k = %s\n" % s.params['split_k'])
+
+
 class epilogueOp(schedOp):
-    """Result write-back: 0 stores 8/16-byte pieces straight from the accumulator registers, 1 parks one MFMA
-    row-tile per wave in a padded LDS strip and streams it out 16 bytes per lane (whole row segments per store).
-    The strips must fit the LDS budget and split into whole wave stores.  Replaces the store stage of the reference's
-    TensorCore template (tensorcoreStoreOp through shared memory, gpu_tensorcore_operator.py), where it is not a choice."""
+    """Result write-back: 0 stores 8/16-byte pieces straight from the accumulator registers; 1 parks one MFMA row-tile
+    per wave in a padded LDS strip as wide as the wave tile and streams it out 16 bytes per lane (whole row segments
+    per store); 2 does the same through strips of half that width, filled twice per row-tile (half the LDS, which is
+    what lets a 256x256 int32 tile keep its stages live in persistent mode).  The strips must fit the LDS budget and
+    split into whole wave stores.  Replaces the store stage of the reference's TensorCore template (tensorcoreStoreOp
+    through shared memory, gpu_tensorcore_operator.py), where it is not a choice."""
 
     def perform(self, s, stage_name, ctx):
         km = ctx.knob_manager
         lds_limit = ctx.getLimit('lds_bytes_per_wg')
-        oes = 2 if s.info['kind'] == 'f16' else 4
-        epi = self.knob(ctx, stage_name, 'epilogue', [0, 1], 1)
-        wtn = self.V(stage_name, 'wave_tile_n')
-        row = self.var(ctx, stage_name, 'epi_row_bytes', 32, 1024, 64)
-        km.addProd([oes, wtn], row)
-        pitch = self.var(ctx, stage_name, 'epi_pitch', 48, 1040, 80)
+        epi = self.knob(ctx, stage_name, 'epilogue', [0, 1, 2], 1)
+        km.addCandidates(epi, [0, 1, 2])
+        oh = epi.replace("P#", "O#")
+        on = self.var(ctx, stage_name, 'epilogue_staged', 0, 1, 1)
+        km.addSUM(1, [on, oh + '_cand0'])
+        # strips per row-tile (1 or 2) and their width in outputs: strips * strip_width = wave_tile_n, whole MFMA tiles each
+        nstr = self.var(ctx, stage_name, 'epi_strips', 1, 2, 1)
+        km.addSUM(nstr, [1, oh + '_cand2'])
+        sw = self.var(ctx, stage_name, 'epi_strip_width', 8, 512, 64)
+        km.addProd([nstr, sw], self.V(stage_name, 'wave_tile_n'))
+        tns = self.var(ctx, stage_name, 'epi_tiles_per_strip', 1, 16, 1)
+        km.addProd([nstr, tns], self.P(stage_name, 'tile_n'))
+        row = self.var(ctx, stage_name, 'epi_row_bytes', 32, 2048, 64)
+        km.addProd([self.V(stage_name, 'out_elem_bytes'), sw], row)
+        pitch = self.var(ctx, stage_name, 'epi_pitch', 48, 2064, 80)
         km.addSUM(pitch, [row, 16])
         lanes = self.var(ctx, stage_name, 'epi_rows_all', 16, 512, 32)
         km.addProd([self.V(stage_name, 'waves'), self.P(stage_name, 'mfma')], lanes)
-        strips = self.var(ctx, stage_name, 'epi_strip_bytes', 768, lds_limit * 4, 768)
+        strips = self.var(ctx, stage_name, 'epi_strip_bytes', 768, lds_limit * 8, 768)
         km.addProd([lanes, pitch], strips)
         base = 0
         if s.info['kind'] != 'f16':
-            base = self.var(ctx, stage_name, 'epi_base', 1024, 2048, 1024)       # column sums, rounded up to 1 KiB
-            kb = self.var(ctx, stage_name, 'epi_base_kib', 1, 2, 1)
+            # column sums of B: one row of block_n sums per wave row, rounded up to 1 KiB
+            base = self.var(ctx, stage_name, 'epi_base', 1024, 16384, 1024)
+            kb = self.var(ctx, stage_name, 'epi_base_kib', 1, 16, 1)
             km.addProd([1024, kb], base)
             bn4 = self.var(ctx, stage_name, 'block_n_bytes4', 64, 2048, 64)
             km.addProd([4, self.V(stage_name, 'block_n')], bn4)
-            km.addLE(bn4, base)
-            slack = self.var(ctx, stage_name, 'block_n_bytes4_plus_1023', 1087, 3071, 1087)
-            km.addSUM(slack, [bn4, 1023])
+            sums = self.var(ctx, stage_name, 'column_sum_bytes', 64, 16384, 64)
+            km.addProd([self.P(stage_name, 'wave_m'), bn4], sums)
+            km.addLE(sums, base)
+            slack = self.var(ctx, stage_name, 'column_sum_bytes_plus_1023', 1087, 17407, 1087)
+            km.addSUM(slack, [sums, 1023])
             km.addLE(base, slack)                               # base is the smallest whole KiB that holds the sums
-        need = self.var(ctx, stage_name, 'epi_lds_needed', 768, lds_limit * 4 + 2048, 768)
+        need = self.var(ctx, stage_name, 'epi_lds_needed', 768, lds_limit * 8 + 16384, 768)
         km.addSUM(need, [strips, base])
         used = self.var(ctx, stage_name, 'epi_lds_bytes', 0, lds_limit, 0)
-        km.addProd([epi, need], used)                       # 0 when the register epilogue is chosen
+        km.addProd([on, need], used)                        # 0 when the register epilogue is chosen
+        # window mode: the region takes the place of the window (dynamic LDS) next to the filter stages
+        ew = self.var(ctx, stage_name, 'epi_lds_bytes_in_window', 0, lds_limit, 0)
+        km.addProd([self.P(stage_name, 'conv_window'), used], ew)
+        tot = self.var(ctx, stage_name, 'lds_bytes_with_epi_in_window', 2048, lds_limit, 4096)
+        km.addSUM(tot, [self.V(stage_name, 'lds_bytes'), ew])
         # a strip must split into whole 1 KiB wave stores: mfma * row_bytes = 1024 * q
-        area = self.var(ctx, stage_name, 'epi_strip_area', 512, 32768, 1024)
+        area = self.var(ctx, stage_name, 'epi_strip_area', 512, 65536, 1024)
         km.addProd([self.P(stage_name, 'mfma'), row], area)
-        area_e = self.var(ctx, stage_name, 'epi_strip_area_used', 0, 32768, 0)
-        km.addProd([epi, area], area_e)
-        q = self.var(ctx, stage_name, 'epi_wave_stores', 0, 32, 0)
+        area_e = self.var(ctx, stage_name, 'epi_strip_area_used', 0, 65536, 0)
+        km.addProd([on, area], area_e)
+        q = self.var(ctx, stage_name, 'epi_wave_stores', 0, 64, 0)
         km.addProd([1024, q], area_e)
         s.params['epilogue'] = km.get_val(epi)
         ctx.addSchedDesc("epilogue = %s\n" % s.params['epilogue'])
@@ -427,7 +459,7 @@ class persistentOp(schedOp):
     """Launch shape: 0 = one output tile per workgroup, 1 = as many workgroups as the device holds at once, each
     walking several output tiles with the k-tiles of all of them in one stream through the LDS stages, so the next
     tile's fetches overlap the current tile's stores.  Needs the LDS-staged epilogue in its own LDS region (the
-    stages stay live), no input window, no L2 prefetch, and the epilogue's store instructions must fit the
+    stages stay live), no input window, no split-K, an even number of k-steps per tile, and the epilogue's store instructions must fit the
     vector-memory counter together with the fetches issued behind them.  No counterpart in the reference (TVM
     launches one thread block per output tile)."""
 
@@ -435,12 +467,14 @@ class persistentOp(schedOp):
         km = ctx.knob_manager
         lds_limit = ctx.getLimit('lds_bytes_per_wg')
         pers = self.knob(ctx, stage_name, 'persistent', [0, 1], 0)
-        km.addLE(pers, self.P(stage_name, 'epilogue'))
+        km.addLE(pers, self.V(stage_name, 'epilogue_staged'))
         pw = self.var(ctx, stage_name, 'persistent_plus_window', 0, 1, 0)
         km.addSUM(pw, [pers, self.P(stage_name, 'conv_window')])
-        if s.info['operator'] == 'gemm':
-            pp = self.var(ctx, stage_name, 'persistent_plus_prefetch', 0, 1, 0)
-            km.addSUM(pp, [pers, self.V(stage_name, 'l2_prefetch_on')])
+        ps1 = self.var(ctx, stage_name, 'persistent_plus_split', 0, 1, 0)
+        km.addSUM(ps1, [pers, self.V(stage_name, 'split_k_on')])
+        # the register buffers must be back in phase at the end of every k-tile: an even number of k-steps
+        po = self.var(ctx, stage_name, 'persistent_plus_single_step', 0, 1, 0)
+        km.addSUM(po, [pers, "O#" + self.V(stage_name, 'k_steps') + '_cand0'])
         pe = self.var(ctx, stage_name, 'persistent_epi_bytes', 0, lds_limit, 0)
         km.addProd([pers, self.V(stage_name, 'epi_lds_needed')], pe)
         tot = self.var(ctx, stage_name, 'lds_bytes_persistent', 2048, lds_limit, 4096)
@@ -450,7 +484,7 @@ class persistentOp(schedOp):
         fl = self.var(ctx, stage_name, 'fetches_behind_stores', 0, 63, 0)
         km.addProd([a2, self.V(stage_name, 'loads_per_tile')], fl)
         st = self.var(ctx, stage_name, 'stores_per_tile', 0, 512, 0)
-        km.addProd([self.P(stage_name, 'tile_m'), self.V(stage_name, 'epi_wave_stores')], st)
+        km.addProd([self.P(stage_name, 'tile_m'), self.V(stage_name, 'epi_strips'), self.V(stage_name, 'epi_wave_stores')], st)
         ps = self.var(ctx, stage_name, 'persistent_stores', 0, 63, 0)
         km.addProd([pers, st], ps)
         vm = self.var(ctx, stage_name, 'persistent_vmem_in_flight', 0, 63, 0)
@@ -461,13 +495,22 @@ class persistentOp(schedOp):
 
 class rasterOp(schedOp):
     """Launch-time tile raster: workgroups are spread over the 8 XCDs and walk the tile grid in column
-    groups of ``group_m`` row-tiles so that one XCD's L2 holds a compact block of A and B."""
+    groups of ``group_m`` row-tiles so that one XCD's L2 holds a compact block of A and B.  Also the issue-order
+    style of a k-step: 1 pins the template's own interleaving of fragment reads, tile loads and MFMAs with scheduling
+    fences, 0 leaves it to the compiler under group hints (what TVM's generated code leaves to NVCC); and how far the
+    wave loads of the next k-tile are spread over the MFMA rows of the step that issues them (0 = all right behind
+    the barrier ... 3 = all rows but the last two): the workgroups of an XCD reach that barrier together, so spreading
+    smooths the demand on the L2."""
 
     def perform(self, s, stage_name, ctx):
         km = ctx.knob_manager
         gm = self.knob(ctx, stage_name, 'raster_group_m', [1, 2, 4, 8, 16, 32], 8)
+        sc = self.knob(ctx, stage_name, 'issue_order', [0, 1], 1)
+        sp = self.knob(ctx, stage_name, 'load_spread', [0, 1, 2, 3], 2)
         s.params['group_m'] = km.get_val(gm)
-        ctx.addSchedDesc("raster group_m = %s\n" % s.params['group_m'])
+        s.params['sched'] = km.get_val(sc)
+        s.params['load_spread'] = km.get_val(sp)
+        ctx.addSchedDesc("raster group_m = %s, issue order = %s\n" % (s.params['group_m'], s.params['sched']))
 
 
 class finishOp(schedOp):
@@ -486,6 +529,7 @@ all_op_methods = {
     'ldsStage': ldsStageOp,
     'ldsSwizzle': ldsSwizzleOp,
     'registerBudget': registerBudgetOp,
+    'splitK': splitKOp,
     'epilogue': epilogueOp,
     'persistent': persistentOp,
     'raster': rasterOp,
@@ -493,7 +537,7 @@ all_op_methods = {
 }
 
 RULE_ORDER = ['start', 'mfmaShape', 'tileWave', 'tileBlock', 'tileK', 'convWindow', 'loadVector', 'ldsStage', 'ldsSwizzle',
-              'registerBudget', 'epilogue', 'persistent', 'raster', 'finish']
+              'registerBudget', 'splitK', 'epilogue', 'persistent', 'raster', 'finish']
 
 
 def sched_via_rule(ctx, s):

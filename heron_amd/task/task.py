@@ -1,9 +1,9 @@
-"""Task: one operator instance to tune - API of the reference's task/task.py:13-103.
+"""Task: one operator instance to tune.
 
-``make_stage_schedules`` builds the template and its constraint system, ``instantiate`` replays
-the recorded schedule steps with a solved KnobManager into a concrete template instance,
-``apply_best`` loads the best row of a records file, ``set_verify_func`` arms the result check
-of the measurer.
+Keeps the interface of the reference's task/task.py:13-103 - ``make_stage_schedules`` (build the template and its
+constraint system), ``instantiate`` (replay the recorded schedule steps with a solved KnobManager into a concrete
+template instance), ``apply_best`` (the best row of a records file), ``apply_sample``, ``set_verify_func`` (arms the
+measurer's result check), ``getStmt`` - on top of a fixed HIP template instead of TVM loop nests.
 """
 import json
 import os
@@ -15,89 +15,97 @@ from ..schedule.sched_op import TemplateSchedule, get_op_methods, sched_via_rule
 
 class Task:
     def __init__(self, name, opfunc, args, target, target_host=None):
-        self.name = name
-        self.args = args
-        self.opfunc = opfunc
-        self.target = target
-        self.target_host = target_host
-        self.build_kwargs = None
-        self.knob_manager = KnobManager()
-        self.not_verify_correctness = True
-        self.ref_input = None
-        self.ref_output = None
-        self.rtol = 0.1
+        self.name, self.opfunc, self.args = name, opfunc, args
+        self.target, self.target_host = target, target_host
         self.config = None
+        self.build_kwargs = None
         self.device_id = 0
+        self.knob_manager = KnobManager()
         self.sched_desc = ""
+        self.template_info = None           # operator / element kind / GEMM view, known once the template is built
+        # result check of the measurer (off until set_verify_func is called, as in the reference)
+        self.not_verify_correctness = True
+        self.ref_input = self.ref_output = None
+        self.rtol = 0.1
 
     def code(self):
         return self.name
 
-    def _context(self, knob_manager):
-        return buildContext(self.config.codegen_type, knob_manager, self.build_kwargs, str(self.target))
-
-    def apply_best(self, path):
-        if self.knob_manager.sched_tups == []:
-            self.make_stage_schedules()
-        to_sort = []
-        for row in open(path):
-            if not row.strip():
-                continue
-            json_dict = json.loads(row)
-            to_sort.append((json_dict['perf'], json_dict['param']))
-        sorted_pairs = sorted(to_sort, key=lambda x: -x[0])
-        # a record written before a knob was added to the template lacks that knob: it then takes its default (off)
-        param = {name: var.defv for name, var in self.knob_manager.solver.vals.items()}
-        param.update(sorted_pairs[0][1])
-        self.knob_manager.solved_knob_vals_phenotype = param
-        self.knob_manager.runtime_perf = sorted_pairs[0][0]
-        self.knob_manager.is_building = False
-        return self.instantiate(self.knob_manager)
-
-    def apply_sample(self, sample):
-        """Instantiate from a measured sample (the reference's version reads an undefined name)."""
-        self.knob_manager.solved_knob_vals_phenotype = dict(sample.knob_manager.solved_knob_vals_phenotype)
-        self.knob_manager.runtime_perf = sample.perf
-        self.knob_manager.is_building = False
-        return self.instantiate(self.knob_manager)
+    # ------------------------------------------------------------------ template and constraint system
+    def _declare(self, knob_manager):
+        """Runs the operator definition under a fresh context; returns (context, schedule object, output tensors)."""
+        ctx = buildContext(self.config.codegen_type, knob_manager, self.build_kwargs, str(self.target))
+        outs = self.opfunc(ctx, *self.args)
+        sched = TemplateSchedule(outs, ctx.tensorize_info)
+        ctx.init_tensor_dict(outs)
+        return ctx, sched, outs
 
     def getOut(self):
-        ctx = self._context(self.knob_manager)
-        return self.opfunc(ctx, *self.args)
+        return self._declare(self.knob_manager)[2]
 
     def make_stage_schedules(self):
-        ctx = self._context(self.knob_manager)
         print(self.args)
-        outs = self.opfunc(ctx, *self.args)
-        s = TemplateSchedule(outs, ctx.tensorize_info)
-        ctx.init_tensor_dict(outs)
-        sched_via_rule(self.config.codegen_type, ctx, s)
+        ctx, sched, _ = self._declare(self.knob_manager)
+        sched_via_rule(self.config.codegen_type, ctx, sched)
         self.sched_desc = ctx.sched_desc
+        self.template_info = ctx.tensorize_info
         self.knob_manager.is_building = False
-        valid, _ = self.knob_manager.solver.solve({}, {})
+        feasible, _ = self.knob_manager.solver.solve({}, {})
         self.dump_constraints()
-        assert valid, "the template has no feasible instance for this shape"
+        if not feasible:
+            raise AssertionError("the template has no feasible instance for this shape")
 
     def dump_constraints(self):
         log_dir = getattr(self.config, "log_dir", None)
-        if not log_dir or not os.path.isdir(log_dir):
-            return
-        with open(os.path.join(log_dir, 'constraints.py'), 'w') as f:
-            f.write(self.knob_manager.solver.dump())
+        if log_dir and os.path.isdir(log_dir):
+            with open(os.path.join(log_dir, 'constraints.py'), 'w') as out:
+                out.write(self.knob_manager.solver.dump())
 
     def instantiate(self, knob_manager):
-        ctx = self._context(knob_manager)
-        outs = self.opfunc(ctx, *self.args)
-        s = TemplateSchedule(outs, ctx.tensorize_info)
-        ctx.init_tensor_dict(outs)
-        args = ctx.input_tensors + outs
-        op_methods = get_op_methods(self.config.codegen_type)
-        for act_name, stage_name in knob_manager.sched_tups:
-            op_methods[act_name](act_name).perform(s, stage_name, ctx)
-        ctx.pos_process(s)
+        """(template schedule, argument tensors) of the point ``knob_manager`` holds."""
+        ctx, sched, outs = self._declare(knob_manager)
+        methods = get_op_methods(self.config.codegen_type)
+        for action, stage in knob_manager.sched_tups:
+            methods[action](action).perform(sched, stage, ctx)
+        ctx.pos_process(sched)
         knob_manager.sched_desc = ctx.sched_desc
-        return s, args
+        return sched, ctx.input_tensors + outs
 
+    # ------------------------------------------------------------------ points from records and samples
+    def _instantiate_values(self, values, perf):
+        km = self.knob_manager
+        km.solved_knob_vals_phenotype = values
+        km.runtime_perf = perf
+        km.is_building = False
+        return self.instantiate(km)
+
+    def apply_best(self, path):
+        """Instantiates the best-performing row of a records file."""
+        if not self.knob_manager.sched_tups:
+            self.make_stage_schedules()
+        rows = [json.loads(line) for line in open(path) if line.strip()]
+        best = max(rows, key=lambda r: r['perf'])
+        # a record written before a knob was added to the template lacks that knob: it then takes its default
+        values = {name: var.defv for name, var in self.knob_manager.solver.vals.items()}
+        values.update(best['param'])
+        return self._instantiate_values(values, best['perf'])
+
+    def apply_sample(self, sample):
+        """Instantiates a measured sample (the reference's version reads an undefined name, task/task.py:45-49)."""
+        return self._instantiate_values(dict(sample.knob_manager.solved_knob_vals_phenotype), sample.perf)
+
+    # ------------------------------------------------------------------ cost-model features
+    def featurize(self, values, own_shape=True):
+        """Compact feature vector of a solved point, or None when the operator set defines none.  ``own_shape=False``:
+        the point belongs to another task of the same operator (a record of an earlier run) and is described with
+        that task's extents."""
+        if self.template_info is None or self.config is None or self.config.codegen_type != 'GPU_MFMA':
+            return None
+        from ..schedule.sched_op.mfma_features import featurize, view_of_values
+        info = self.template_info if own_shape else view_of_values(self.template_info, values)
+        return featurize(info, values)
+
+    # ------------------------------------------------------------------ verification and text form
     def set_verify_func(self, func, rtol=0.1):
         self.rtol = rtol
         self.not_verify_correctness = False
@@ -107,8 +115,8 @@ class Task:
 
     def getStmt(self, knob_manager):
         """Text form of an instance (the reference returns the lowered TIR here)."""
-        s, args = self.instantiate(knob_manager)
-        lines = ["%s %s" % (s.info['operator'], s.info['kind'])]
+        sched, args = self.instantiate(knob_manager)
+        lines = ["%s %s" % (sched.info['operator'], sched.info['kind'])]
         lines += ["  %s: %s %s" % (t.name, t.shape, t.dtype) for t in args]
-        lines.append("  template: " + s.describe())
+        lines.append("  template: " + sched.describe())
         return "\n".join(lines)

@@ -20,7 +20,10 @@ class GATuner(Tuner):
     def optimize(self, env, population, stat, s_time):
         all_pop = [] + population
         for _ in range(self.config.iter_walks):
-            if hasattr(self.cost_model, 'bst') and self.cost_model.bst is None:
+            # nothing measured yet: the reference has no fitness to evolve on (ga_tuner.py:16-17); with an analytic
+            # estimate of the template the walks evolve on that, so the first measured batch is already a good one
+            if hasattr(self.cost_model, 'bst') and self.cost_model.bst is None and \
+                    not getattr(self.cost_model, 'has_prior', False):
                 break
             self.inferKeyVariables(env, population)
             population = self.RankPop(population)

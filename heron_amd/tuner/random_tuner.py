@@ -1,33 +1,35 @@
-"""Constrained-random baselines (tuner/random_tuner.py:6-27 of the reference)."""
+"""Baselines without a search operator: every walk draws a fresh batch of constrained-random samples.
+
+``CRandTuner`` lets the cost model rank what it drew (the batch plus the 20 best-predicted points seen so far go on to
+selection); ``CRandSampler`` ignores the model altogether (all predictions zeroed), i.e. pure constrained-random
+search.  Same roles as the two classes of the reference's tuner/random_tuner.py:6-27."""
 from .tuner import Tuner
 
 
-class CRandTuner(Tuner):
+class _ConstrainedRandom(Tuner):
+    use_model = True
+
     def check_feasible_exits(self, env, num=1e3):
-        return
+        return              # constrained sampling needs no per-knob feasible sets
 
     def optimize(self, env, pop, stat, s_time):
-        samples = [] + pop
-        population = []
+        seen = list(pop)
+        batch = []
         for _ in range(self.config.iter_walks):
-            population = self.constrained_random_sample(env, self.config.pop_num)
-            samples = samples + population
-            self.recordStat(samples, env, s_time, stat)
-        population += sorted(samples, key=lambda x: -x.predict)[:20]
-        return population, samples
+            batch = self.constrained_random_sample(env, self.config.pop_num)
+            seen += batch
+            if not self.use_model:
+                for sample in seen:
+                    sample.predict = 0
+            self.recordStat(seen, env, s_time, stat)
+        if self.use_model:
+            batch = batch + sorted(seen, key=lambda s: s.predict, reverse=True)[:20]
+        return batch, seen
 
 
-class CRandSampler(Tuner):
-    def check_feasible_exits(self, env, num=1e3):
-        return
+class CRandTuner(_ConstrainedRandom):
+    use_model = True
 
-    def optimize(self, env, pop, stat, s_time):
-        samples = [] + pop
-        population = []
-        for _ in range(self.config.iter_walks):
-            population = self.constrained_random_sample(env, self.config.pop_num)
-            samples = samples + population
-            for sample in samples:
-                sample.predict = 0
-            self.recordStat(samples, env, s_time, stat)
-        return population, samples
+
+class CRandSampler(_ConstrainedRandom):
+    use_model = False

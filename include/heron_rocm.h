@@ -73,16 +73,23 @@ typedef struct hrn_kernel_desc {
     int32_t mfma;       /* 32 -> 32x32x(16 f16|32 i8), 16 -> 16x16x(32 f16|64 i8) */
     int32_t stages;     /* LDS stages of the A/B tiles, 2..5 (2 = double buffer) */
     int32_t swizzle;    /* LDS 16-byte-chunk XOR swizzle: 0 none, 1 row, 2 row/2, 3 row/4 */
-    int32_t epilogue;   /* 0 = store accumulators straight from registers, 1 = stage C through LDS */
+    int32_t epilogue;   /* 0 = store accumulators straight from registers, 1 = stage C through LDS strips as wide as
+                           the wave tile, 2 = through strips of half that width (half the LDS) */
     int32_t waves_per_eu; /* 0 = let the compiler pick, else occupancy hint 1..4 */
-    int32_t l2_prefetch;  /* 0 = off, d = touch the cache lines of the k-tile d tiles past the one being fetched */
-    int32_t ablate;       /* diagnostic switches of the template; must be 0 for correct results */
-    int32_t load_mode;    /* 0 = global -> LDS directly, 1 = global -> registers -> LDS with two tiles in flight (stages must be 2) */
     int32_t conv_window;  /* conv2d only: 1 = keep the reachable input window in LDS and read every filter tap from it
                              (needs stride 1, dilation 1, 'same' padding, CI*2 a multiple of bkb) instead of im2col tiles */
     int32_t persistent;   /* 1 = launch only as many workgroups as fit the device and let each walk several output tiles,
                              fetching the next tile's operands while the current result is stored (needs epilogue 1 and
                              N*out_bytes a multiple of 16) */
+    int32_t split_k;      /* 1 = K is cut into hrn_problem.split_k slices that run as separate workgroups; the kernel
+                             stores raw fp32 / int32 partial sums per slice into hrn_problem.workspace and a second
+                             pass of the library adds them into C (for small M*N with long K: more workgroups than
+                             output tiles).  Not with persistent or conv_window. */
+    int32_t sched;        /* issue order of a k-step: 1 = the template's own interleaving of fragment reads, tile loads
+                             and MFMAs is pinned with scheduling fences, 0 = left to the compiler under group hints */
+    int32_t load_spread;  /* with sched = 1: how far the wave loads of the next k-tile are spread over the MFMA rows of the
+                             step that issues them: 0 = all right behind the barrier, 1 = over a quarter of the rows,
+                             2 = half, 3 = all but the last two (smoother demand on the L2, later arrival) */
 } hrn_kernel_desc;
 
 /* Resource usage of a built instance, for cross-checks of the constraint set. */
@@ -116,6 +123,12 @@ typedef struct hrn_problem {
     /* launch-time raster knob: tiles are walked in column groups of this many row-tiles */
     int32_t group_m;
     int32_t cstride_w, cpad_w, cdil_w;
+    /* split-K instances only (hrn_kernel_desc.split_k = 1): number of K slices wanted (>= 1; slices never get less
+     * than one k-tile, so fewer may run) and the caller-owned device workspace for the partial sums, at least
+     * hrn_splitk_workspace_bytes() large and 16-byte aligned.  Launches that share a workspace must not overlap. */
+    int32_t split_k;
+    void* workspace;
+    size_t workspace_bytes;
 } hrn_problem;
 
 typedef struct hrn_module hrn_module;
@@ -202,6 +215,14 @@ int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, co
  */
 int hrn_probe_mfma(int dtype, int mfma, int random_operands, double* tops_out, void* stream);
 int hrn_probe_copy(const void* src, void* dst, size_t bytes, int repeat, double* gbs_out, void* stream);
+
+/*
+ * Bytes of workspace a launch of `desc` on problem `p` (with p->split_k set) needs: slices * batch * m * n * 4, or 0
+ * when the instance is not a split-K one; negative HRN_E_* on bad arguments.  The reference has no counterpart: its
+ * TensorCore schedules never split the reduction over thread blocks (ops/cuda/dense.py:18-26 binds only the
+ * spatial axes to blockIdx).
+ */
+int64_t hrn_splitk_workspace_bytes(const hrn_kernel_desc* desc, const hrn_problem* p);
 
 /* Fills an hrn_problem for the plain cases (packed row-major operands). */
 void hrn_problem_gemm(hrn_problem* p, int batch, int m, int n, int k);

@@ -22,7 +22,10 @@ from heron_amd.task.task import Task                                  # noqa: E4
 
 TASKS = [("gemm", [2048, 1024, 2048], "float16", 8), ("gemm", [2048, 1024, 2048], "int8", 8),
          ("bmm", [8, 512, 256, 512], "float16", 4), ("c2d", [4, 28, 28, 64, 128, 3, 3, 1, 1, 1], "float16", 8),
-         ("c2d", [4, 28, 28, 64, 128, 3, 3, 1, 1, 1], "int8", 6), ("c2d", [2, 30, 30, 32, 64, 3, 3, 2, 1, 1], "float16", 4)]
+         ("c2d", [4, 28, 28, 64, 128, 3, 3, 1, 1, 1], "int8", 6), ("c2d", [2, 30, 30, 32, 64, 3, 3, 2, 1, 1], "float16", 4),
+         # few output tiles and a long K: the split-K part of the space
+         ("gemm", [256, 4096, 512], "float16", 5), ("gemm", [128, 8192, 256], "int8", 5),
+         ("c2d", [16, 7, 7, 512, 512, 3, 3, 1, 1, 1], "float16", 4)]
 
 if __name__ == "__main__":
     random.seed(20240607)
@@ -44,7 +47,8 @@ if __name__ == "__main__":
             if not valid or not B.check_desc(d) or tup in seen:
                 continue
             seen.add(tup)
-            out.append({"desc": list(tup), "group_m": int(s.params["group_m"]), "from": [op, shape, dtype]})
+            out.append({"desc": list(tup), "group_m": int(s.params["group_m"]), "split_k": int(s.params["split_k"]),
+                        "from": [op, shape, dtype]})
             got += 1
     with open(os.path.join(HERE, "fuzz_instances.json"), "w") as f:
         json.dump(out, f, indent=0)

@@ -25,11 +25,38 @@ def test_header_symbols_exported_and_bound():
     assert b"gfx950" in B.lib().hrn_version()
 
 
-def test_struct_sizes_match_header_layout():
+def header_struct(name):
+    """(field name, C type, array length) of every member of ``struct name`` in the header, in declaration order."""
+    text = open(os.path.join(ROOT, "include", "heron_rocm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (name, name), text, flags=re.S).group(1)
+    out = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        ctype, names = re.match(r"((?:u?int\d+_t|size_t|char|void\s*\*))\s*(.*)", decl, flags=re.S).groups()
+        for n in names.split(","):
+            m = re.match(r"\s*(\w+)(?:\[(\d+)\])?\s*$", n)
+            out.append((m.group(1), ctype.replace(" ", ""), int(m.group(2) or 0)))
+    return out
+
+
+C_TYPES = {"int32_t": ctypes.c_int32, "int64_t": ctypes.c_int64, "uint64_t": ctypes.c_uint64, "size_t": ctypes.c_size_t,
+           "void*": ctypes.c_void_p, "char": ctypes.c_char}
+
+
+def test_struct_layouts_match_header():
+    """Every ctypes structure has the header's members, in the header's order, with the header's types."""
+    for name, cls in (("hrn_kernel_desc", B.KernelDesc), ("hrn_kernel_info", B.KernelInfo), ("hrn_problem", B.Problem),
+                      ("hrn_devinfo", B.DevInfo)):
+        want = [(n, C_TYPES[t] * k if k else C_TYPES[t]) for n, t, k in header_struct(name)]
+        have = [(n, t) for n, t in cls._fields_]
+        assert [n for n, _ in have] == [n for n, _ in want], name
+        for (n, th), (_, tw) in zip(have, want):
+            assert ctypes.sizeof(th) == ctypes.sizeof(tw) and th._type_ == tw._type_, (name, n)
     assert ctypes.sizeof(B.KernelDesc) == 17 * 4
-    assert ctypes.sizeof(B.KernelInfo) == 8 * 4
-    assert ctypes.sizeof(B.Problem) == 8 * 4 + 3 * 8 + 10 * 4 + 4 * 4
-    assert ctypes.sizeof(B.DevInfo) == 64 + 128 + 10 * 4 + 8
+    assert B.KernelDesc.KEYS == tuple(n for n, _ in B.KernelDesc._fields_)
 
 
 def test_check_desc_mirrors_template_constraints():
@@ -37,7 +64,9 @@ def test_check_desc_mirrors_template_constraints():
     assert B.check_desc(ok) and B.lds_bytes(ok) == 131072
     bad = [
         instances.D(instances.F16, instances.GEMM, 256, 256, 128, 2, 2, 32, 3, 2),    # 192 KiB LDS
-        instances.D(instances.F16, instances.GEMM, 256, 256, 64, 2, 2, 16, 2, 0),     # one k-step per tile
+        instances.D(instances.F16, instances.GEMM, 256, 128, 64, 4, 2, 16, 2, 3, epi=1, pers=1),   # persistent with one k-step per tile
+        instances.D(instances.F16, instances.GEMM, 128, 128, 128, 2, 2, 32, 2, 1, epi=1, pers=1, split=1),   # persistent + split-K
+        instances.D(instances.F16, instances.GEMM, 192, 128, 128, 3, 2, 32, 2, 1),    # wave rows not a power of two
         instances.D(instances.F16, instances.GEMM, 96, 128, 128, 2, 2, 32, 2, 0),     # 96 rows / (2 waves x 32)
         instances.D(instances.F16, instances.GEMM, 128, 128, 256, 2, 2, 16, 2, 2),    # swizzle period 32 > mfma 16
         instances.D(instances.F16, instances.GEMM, 128, 128, 128, 2, 2, 32, 2, 1, win=1),   # window mode is a conv load path

@@ -1,6 +1,6 @@
 """GPU parity of template instances drawn from the tuner's own search space (tests/golden/fuzz_instances.json, made by
 tests/golden/make_fuzz_instances.py with a fixed seed): knob combinations nobody picked by hand - odd per-wave tile
-counts, five stages, persistent launches, window mode - against the oracle on ragged shapes.
+counts, five stages, one k-step per tile, persistent launches, window mode, split-K - against the oracle on ragged shapes.
 Integer results bit-exact, fp16 within rel. error 1e-2.
 """
 import json
@@ -13,9 +13,9 @@ import torch
 import oracle
 from heron_amd import backend as B
 from heron_amd import hostops, instances, workloads
+from parity_checks import check_f16
 
 pytestmark = pytest.mark.gpu
-REL_TOL = 1e-2
 HERE = os.path.dirname(os.path.abspath(__file__))
 FUZZ = json.load(open(os.path.join(HERE, "golden", "fuzz_instances.json")))
 
@@ -30,7 +30,7 @@ def dev(a):
 
 def close(got, ref, f16):
     if f16:
-        assert float(np.abs(got.astype(np.float32) - ref).max()) / (float(np.abs(ref).max()) + 1e-30) <= REL_TOL
+        check_f16(got, ref)
     else:
         assert np.array_equal(got, ref)
 
@@ -38,7 +38,7 @@ def close(got, ref, f16):
 @pytest.mark.parametrize("entry", FUZZ, ids=lambda e: "-".join(map(str, e["desc"])))
 def test_sampled_instance(entry, hrn):
     d = B.make_desc(*entry["desc"])
-    gm = entry["group_m"]
+    gm, sk = entry["group_m"], entry["split_k"]
     m = B.Module(d)
     assert m.info["scratch_bytes"] >= 0
     f16 = d.dtype == instances.F16
@@ -48,10 +48,10 @@ def test_sampled_instance(entry, hrn):
             print("fuzz gemm", entry["desc"], (M, K, N), flush=True)
             if f16:
                 A, Bm = workloads.gemm_f16_inputs(M, K, N, seed=200 + i)
-                close(hostops.gemm(m, dev(A), dev(Bm), group_m=gm).cpu().numpy(), oracle.gemm_f32(A, Bm), True)
+                close(hostops.gemm(m, dev(A), dev(Bm), group_m=gm, split_k=sk).cpu().numpy(), oracle.gemm_f32(A, Bm), True)
             else:
                 A, Bm = workloads.gemm_u8s8_inputs(M, K, N, seed=200 + i)
-                close(hostops.gemm(m, dev(A), dev(Bm), group_m=gm).cpu().numpy(), oracle.gemm_int64_numpy(A, Bm), False)
+                close(hostops.gemm(m, dev(A), dev(Bm), group_m=gm, split_k=sk).cpu().numpy(), oracle.gemm_int64_numpy(A, Bm), False)
             ran += 1
     else:
         for i, case in enumerate(CONV_CASES):
@@ -63,10 +63,10 @@ def test_sampled_instance(entry, hrn):
             window_ok = s == 1 and dl == 1 and 2 * p == KH - 1 and (CI * es) % d.bkb == 0
             if d.conv_window and not window_ok:
                 with pytest.raises(B.HeronRocmError):
-                    hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, dl, group_m=gm)
+                    hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, dl, group_m=gm, split_k=sk)
                 continue
             try:
-                Y = hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, dl, group_m=gm).cpu().numpy()
+                Y = hostops.conv2d_nhwc(m, dev(X), dev(Wt), s, p, dl, group_m=gm, split_k=sk).cpu().numpy()
             except B.HeronRocmError as e:
                 assert d.conv_window and "exceeds 163840" in str(e)          # window + static LDS too large for this image width
                 continue

@@ -11,10 +11,10 @@ import torch
 import oracle
 from heron_amd import backend as B
 from heron_amd import hostops, instances, workloads
+from parity_checks import REL_TOL, check_f16
 
 pytestmark = pytest.mark.gpu
 
-REL_TOL = 1e-2          # tolerance stated for fp16 inputs / fp32 accumulate
 _mods = {}
 
 
@@ -27,15 +27,6 @@ def mod_for(desc):
 
 def dev(a):
     return torch.from_numpy(a).cuda()
-
-
-def check_f16(got, ref):
-    got = got.astype(np.float32)
-    scale = float(np.abs(ref).max()) + 1e-30
-    err = float(np.abs(got - ref).max())
-    assert err / scale <= REL_TOL, (err, scale)
-    # element-wise: fp16 rounding of the result (2^-11 relative) + accumulation noise
-    assert np.all(np.abs(got - ref) <= 2e-3 * np.abs(ref) + 2e-3 * scale)
 
 
 GEMM_SHAPES = [(64, 64, 64), (256, 256, 256), (512, 640, 384), (100, 200, 72), (8, 4096, 16), (300, 1024, 520)]
@@ -65,8 +56,8 @@ def test_gemm_f16_within_tolerance(tup, hrn):
 
 
 @pytest.mark.parametrize("desc", instances.variant_descs(), ids=lambda d: "-".join(map(str, d.as_tuple())))
-def test_optional_load_paths(desc, hrn):
-    """L2 prefetch touches and the register-staged load path must not change any result."""
+def test_template_variants(desc, hrn):
+    """LDS-staged epilogue, one k-step per k-tile (alternating register buffers), window and im2col conv load paths."""
     m = mod_for(desc)
     if desc.op == instances.CONV and desc.conv_window:
         same = [(2, 14, 14, 64, 64, 3, 3, 1, 1, 1), (1, 9, 11, 64, 32, 3, 3, 1, 1, 1), (2, 8, 8, 64, 48, 1, 1, 1, 0, 1),
@@ -295,6 +286,80 @@ def test_persistent_rejects_partial_chunks(hrn):
         hostops.gemm(m, dev(A), dev(Bm))
 
 
+@pytest.mark.parametrize("desc", instances.splitk_descs(), ids=lambda d: "-".join(map(str, d.as_tuple())))
+def test_split_k(desc, hrn):
+    """K cut into slices that run as separate workgroups: partial sums + the reduction pass give the one-pass result
+    (uint8 bit-exact, fp16 within 1e-2) for slice counts that divide the k-tiles, that do not, that exceed them, and 1."""
+    m = mod_for(desc)
+    f16 = desc.dtype == instances.F16
+    if desc.op == instances.CONV:
+        cases = [(16, 7, 7, 512, 64, 3, 3, 1, 1, 1), (2, 15, 15, 64, 48, 3, 3, 2, 1, 1), (1, 9, 9, 32, 16, 5, 5, 1, 2, 2)]
+        for i, case in enumerate(cases):
+            N, H, W, CI, CO, KH, KW, st, pd, dl = case
+            gen = workloads.conv2d_inputs if f16 else workloads.conv2d_u8s8_inputs
+            X, Wt = gen(N, H, W, CI, CO, KH, KW, seed=300 + i)
+            ref = oracle.conv2d_nhwc_f32(X, Wt, st, pd, dl) if f16 else oracle.conv2d_nhwc_u8s8s32(X, Wt, st, pd, dl)
+            for split in (1, 2, 3, 8, 64):
+                print("split-k conv", desc.as_tuple(), case, split, flush=True)
+                Y = hostops.conv2d_nhwc(m, dev(X), dev(Wt), st, pd, dl, split_k=split).cpu().numpy()
+                if f16:
+                    check_f16(Y, ref)
+                else:
+                    assert np.array_equal(Y, ref)
+        return
+    for i, (M, K, N) in enumerate([(100, 4096, 72), (784, 4608, 256), (64, 64, 64), (130, 1040, 36)]):
+        if f16:
+            A, Bm = workloads.gemm_f16_inputs(M, K, N, seed=310 + i)
+            ref = oracle.gemm_f32(A, Bm)
+        else:
+            A, Bm = workloads.gemm_u8s8_inputs(M, K, N, seed=310 + i)
+            ref = oracle.gemm_int64_numpy(A, Bm).astype(np.int32)
+        for split in (1, 2, 5, 16, 1000):
+            print("split-k gemm", desc.as_tuple(), (M, K, N), split, flush=True)
+            C = hostops.gemm(m, dev(A), dev(Bm), split_k=split).cpu().numpy()
+            if f16:
+                check_f16(C, ref)
+            else:
+                assert np.array_equal(C, ref)
+    # batched: every batch entry has its own slices
+    if f16:
+        A = np.stack([workloads.gemm_f16_inputs(96, 2048, 40, seed=330 + b)[0] for b in range(3)])
+        Bm = np.stack([workloads.gemm_f16_inputs(96, 2048, 40, seed=330 + b)[1] for b in range(3)])
+        C = hostops.gemm(m, dev(A), dev(Bm), split_k=4).cpu().numpy()
+        for b in range(3):
+            check_f16(C[b], oracle.gemm_f32(A[b], Bm[b]))
+
+
+def test_split_k_error_paths(hrn):
+    """A split-K instance without (or with too small a) workspace, and a slice count on an instance built without
+    split_k, are refused."""
+    d = instances.splitk_descs()[0]
+    m = mod_for(d)
+    A, Bm = workloads.gemm_f16_inputs(64, 1024, 64, seed=1)
+    a, b = dev(A), dev(Bm)
+    c = torch.empty((64, 64), dtype=torch.float16, device="cuda")
+    L = B.lib()
+    p = B.gemm_problem(1, 64, 64, 1024, 8, split_k=4)
+    need = B.splitk_workspace_bytes(d, p)
+    assert need == 4 * 64 * 64 * 4
+    import ctypes
+    assert L.hrn_launch_gemm_f16(m._h, ctypes.byref(p), a.data_ptr(), b.data_ptr(), c.data_ptr(), 0) == B.HRN_E_BADPARAM
+    assert b"workspace" in L.hrn_last_error()
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    p.workspace, p.workspace_bytes = ws.data_ptr(), need - 16
+    assert L.hrn_launch_gemm_f16(m._h, ctypes.byref(p), a.data_ptr(), b.data_ptr(), c.data_ptr(), 0) == B.HRN_E_BADPARAM
+    assert b"too small" in L.hrn_last_error()
+    p.workspace_bytes = need
+    assert L.hrn_launch_gemm_f16(m._h, ctypes.byref(p), a.data_ptr(), b.data_ptr(), c.data_ptr(), 0) == B.HRN_OK
+    torch.cuda.synchronize()
+    check_f16(c.cpu().numpy(), oracle.gemm_f32(A, Bm))
+    plain = mod_for(instances.BEST["small_f16"])
+    with pytest.raises(B.HeronRocmError):
+        hostops.gemm(plain, a, b, split_k=2)
+    p0 = B.gemm_problem(1, 64, 64, 1024, 8)
+    assert B.splitk_workspace_bytes(instances.BEST["small_f16"], p0) == 0
+
+
 def test_conv_1x1_is_gemm(hrn):
     """A 1x1 convolution is the GEMM of the flattened pixels: both templates must agree bit for bit."""
     tup = instances.PARITY_SHAPES[2]
@@ -383,7 +448,8 @@ def test_device_info_and_timing(hrn):
 def test_cold_cache_timing(hrn):
     """Launches timed after a cache flush: the 4 MiB-operand GEMM that lives in L2/MALL when repeated takes longer
     from HBM, and the result is still correct."""
-    m = mod_for(instances.BEST["gemm_f16_4096"])
+    from heron_amd import tuned
+    m = mod_for(tuned.load("gemm_f16_4096").desc)
     A, Bm = workloads.gemm_f16_inputs(2048, 1024, 2048, seed=4)
     a, b = dev(A), dev(Bm)
     c = torch.empty((2048, 2048), dtype=torch.float16, device="cuda")

@@ -96,7 +96,7 @@ def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
     t = Task("t", getOpFromName(op), shape + [dtype, dtype], "rocm")
     t.config = cfg
     t.make_stage_schedules()
-    assert len(t.knob_manager.knob_names) == 14 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
+    assert len(t.knob_manager.knob_names) == 16 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
     seen = set()
     for _ in range(40):
         km = copy.deepcopy(t.knob_manager)
@@ -107,17 +107,20 @@ def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
         g = s.info['gemm_view']
         assert d.bm <= 16 * math.ceil(g['M'] / 16) and d.bn <= 16 * math.ceil(g['N'] / 16)
         vals = km.solved_knob_vals_phenotype
-        lds_key = [k for k in km.solver.vals if k.endswith("VA:lds_bytes_total")] or \
-                  [k for k in km.solver.vals if k.endswith("VA:lds_bytes")]
+        lds_key = [k for k in km.solver.vals if k.endswith("VA:lds_bytes")]
         epi_key = [k for k in km.solver.vals if k.endswith("VA:epi_lds_bytes")][0]
         if d.persistent:                                                       # stages and epilogue region both live
             pkey = [k for k in km.solver.vals if k.endswith("VA:lds_bytes_persistent")][0]
             assert B.lds_bytes(d) == vals[pkey]
-        else:
-            assert B.lds_bytes(d) == max(vals[lds_key[0]], vals[epi_key])     # static LDS; the conv window is dynamic
-        if op == "c2d" and d.conv_window:
+        elif d.conv_window:
+            # static LDS = the filter stages; the window is dynamic LDS and the epilogue region takes its place later
+            assert B.lds_bytes(d) == vals[lds_key[0]]
             win_key = [k for k in km.solver.vals if k.endswith("VA:window_bytes")][0]
-            assert vals[win_key] == (d.bm + 2 * (56 + 1)) * (128 if dtype == "float16" else 64) and B.lds_bytes(d) + vals[win_key] <= 163840 - 1024
+            assert vals[win_key] == (d.bm + 2 * (56 + 1)) * (128 if dtype == "float16" else 64)
+            assert B.lds_bytes(d) + vals[win_key] <= 163840 - 1024 and B.lds_bytes(d) + vals[epi_key] <= 163840
+        else:
+            assert B.lds_bytes(d) == max(vals[lds_key[0]], vals[epi_key])
+        assert (d.split_k == 1) == (s.params['split_k'] > 1)
         assert [a.name for a in args][-1] == s.info['stage_name']
         seen.add(d.as_tuple())
     assert len(seen) > 20
@@ -370,8 +373,12 @@ def test_pretrained_cross_task_model_steers_a_new_task(tmp_path):
     assert len(stat) == 2
     # records of another operator family are refused
     from heron_amd.model import PretrainedCostModel
+    other = tmp_path / "other_family.txt"
+    with open(other, "w") as f:
+        for r in rows[:4]:
+            f.write(json.dumps(dict(r, param={k.replace("ST:dense", "ST:conv2d_nhwc"): v for k, v in r["param"].items()})) + "\n")
     with pytest.raises(ValueError):
-        PretrainedCostModel(env_b.task, env_b.config).fit_from_records([rec_a], 7)
+        PretrainedCostModel(env_b.task, env_b.config).fit_from_records([str(other)], 7)
 
 
 TUNED = os.path.join(os.path.dirname(os.path.abspath(__file__)), "quick_start", "rocm", "tuned")
