@@ -156,10 +156,10 @@ def run_probes(torch, B):
     dst = torch.empty(n, dtype=torch.uint8, device="cuda")
     st = torch.cuda.current_stream().cuda_stream
     out = {
-        "mfma_f16_const_operands_TFLOPs": B.probe_mfma(B.HRN_DT_F16, 16, False, st),
-        "mfma_f16_random_operands_TFLOPs": B.probe_mfma(B.HRN_DT_F16, 16, True, st),
-        "mfma_i8_const_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 16, False, st),
-        "mfma_i8_random_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 16, True, st),
+        "mfma_f16_const_operands_TFLOPs": B.probe_mfma(B.HRN_DT_F16, 32, False, st),
+        "mfma_f16_random_operands_TFLOPs": B.probe_mfma(B.HRN_DT_F16, 32, True, st),
+        "mfma_i8_const_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 32, False, st),
+        "mfma_i8_random_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 32, True, st),
         "hbm_copy_1GiB_read_plus_write_GBs": B.probe_copy(src.data_ptr(), dst.data_ptr(), n, 10, st),
     }
     del src, dst

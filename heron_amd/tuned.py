@@ -5,6 +5,8 @@
 ``Task.apply_best`` - the same path ``run.py -t`` takes - and returns the template descriptor, its launch-time
 parameters and the record it came from.  The benchmark, smoke and the full-size GPU tests all run these instances.
 """
+import contextlib
+import io
 import json
 import math
 import os
@@ -46,7 +48,8 @@ def load(name):
     cfg.codegen_type, cfg.target_name = 'GPU_MFMA', 'rocm'
     task = Task(name, getOpFromName(op), shape + [dtype, dtype], "rocm")
     task.config = cfg
-    sched, _ = task.apply_best(path)
+    with contextlib.redirect_stdout(io.StringIO()):      # building the template prints the task's arguments
+        sched, _ = task.apply_best(path)
     best = max((json.loads(line) for line in open(path) if line.strip()), key=lambda r: r["perf"])
     inst = TunedInstance(name, sched.to_desc(), int(sched.params['group_m']), int(sched.params.get('split_k', 1)),
                          best["code"], math.exp(-best["perf"]), path, dict(sched.params))
