@@ -17,6 +17,7 @@ HRN_DT_F16, HRN_DT_U8S8 = 0, 1
 HRN_OP_GEMM, HRN_OP_CONV2D = 0, 1
 HRN_OK = 0
 HRN_E_BADPARAM, HRN_E_BUILD, HRN_E_LOAD, HRN_E_LAUNCH, HRN_E_TIMEOUT, HRN_E_NODEVICE = -1, -2, -3, -4, -5, -6
+STATIC_WORKSPACE_BYTES = 32 << 20      # HRN_STATIC_WORKSPACE_BYTES
 
 # flags every HIP translation unit of this package is compiled with
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -131,6 +132,7 @@ SYMBOLS = {
     "hrn_launch_conv2d_nhwc_f16": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
     "hrn_launch_bmm_u8s8": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
     "hrn_launch_conv2d_nhwc_u8s8": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
+    "hrn_launch_splitk_static": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp]),
     "hrn_launch_repeat": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _vp]),
     "hrn_time": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _i, _i, _d, ctypes.POINTER(_d), _vp]),
     "hrn_time_cold": (_i, [_vp, ctypes.POINTER(Problem), _vp, _vp, _vp, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
@@ -275,6 +277,10 @@ class Module:
     def launch(self, problem, a_ptr, b_ptr, c_ptr, stream=0):
         self.bind_workspace(problem)
         _check(self._launcher(problem)(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, stream))
+
+    def launch_splitk_static(self, problem, a_ptr, b_ptr, c_ptr, stream=0):
+        """Split-K launch whose partial sums live in the library's own static device workspace (no allocation)."""
+        _check(lib().hrn_launch_splitk_static(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, stream))
 
     def launch_repeat(self, problem, a_ptr, b_ptr, c_ptr, count, stream=0):
         """``count`` back-to-back launches issued from one host call."""

@@ -20,6 +20,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <fstream>
+#include <mutex>
 #include <sstream>
 #include <string>
 #include <thread>
@@ -501,6 +502,34 @@ int run_plan(const hrn_module* mod, const hrn_problem* p, const LaunchPlan& plan
     return HRN_OK;
 }
 
+// ---- split-K workspace that needs no allocation --------------------------------------------------------------
+// Device memory every GPU the library runs on holds until the process ends; hrn_launch_splitk_static keeps the
+// partial sums of a split-K launch here instead of in a caller-owned workspace.  In host code the array's name is
+// only a stand-in: its device address is looked up once per device and that pointer is what kernels get.
+static __device__ __align__(256) unsigned char scratch[HRN_STATIC_WORKSPACE_BYTES];
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];
+bool g_scratch_known[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+// address of `scratch` on the current device (looked up on the first call per device)
+int static_scratch(void** out) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(HRN_E_BADPARAM, "device index %d", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_known[dev]) {
+        void* ptr = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(HRN_E_LAUNCH, "hipGetSymbolAddress returned a null address");
+        g_scratch_ptr[dev] = ptr;
+        g_scratch_known[dev] = true;
+    }
+    *out = g_scratch_ptr[dev];
+    return HRN_OK;
+}
+
 int launch(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream) {
     LaunchPlan plan;
     int rc = fill_args(mod, p, A, B, C, p ? p->workspace : nullptr, p ? p->workspace_bytes : 0, &plan);
@@ -801,6 +830,25 @@ int hrn_launch_repeat(const hrn_module* mod, const hrn_problem* p, const void* A
         if (rc) return rc;
     }
     return HRN_OK;
+}
+
+int hrn_launch_splitk_static(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream) {
+    if (!mod || !p) return fail(HRN_E_BADPARAM, "null argument");
+    if (!mod->desc.split_k) return fail(HRN_E_BADPARAM, "hrn_launch_splitk_static needs an instance built with split_k");
+    if (p->m <= 0 || p->n <= 0 || p->k <= 0 || p->batch <= 0 || p->split_k < 1) return fail(HRN_E_BADPARAM, "empty problem or split_k < 1");
+    int kps, split;
+    split_shape(mod->desc, p, &kps, &split);
+    const int64_t need = splitk_bytes(p, split);
+    if (need > (int64_t)HRN_STATIC_WORKSPACE_BYTES)
+        return fail(HRN_E_BADPARAM, "split-K partial sums of %lld bytes (%d slices x %d x %d x %d x 4) exceed the library's static workspace of %lld bytes",
+                    (long long)need, split, p->batch, p->m, p->n, (long long)HRN_STATIC_WORKSPACE_BYTES);
+    void* ws = nullptr;
+    int rc = static_scratch(&ws);
+    if (rc) return rc;
+    LaunchPlan plan;
+    rc = fill_args(mod, p, A, B, C, ws, (size_t)HRN_STATIC_WORKSPACE_BYTES, &plan);
+    if (rc) return rc;
+    return run_plan(mod, p, plan, ws, (hipStream_t)stream);
 }
 
 int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, int number, int repeat,

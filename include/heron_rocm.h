@@ -181,6 +181,19 @@ int hrn_launch_conv2d_nhwc_f16(const hrn_module* mod, const hrn_problem* p, cons
 int hrn_launch_bmm_u8s8(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
 int hrn_launch_conv2d_nhwc_u8s8(const hrn_module* mod, const hrn_problem* p, const void* In, const void* Filter, void* Out, void* stream);
 
+/*
+ * Split-K launch that allocates nothing.  No counterpart in the reference; it is for callers that cannot allocate
+ * device memory around a launch (code under HIP graph capture, tight serving loops, harnesses that forbid it).  Same as
+ * launching a split_k instance through the entry points above, except that the partial sums go to a workspace that
+ * is part of the library's own device image (HRN_STATIC_WORKSPACE_BYTES per GPU, held until the process ends) instead
+ * of hrn_problem.workspace, which is ignored.  A problem whose partial sums (slices * batch * m * n * 4 bytes) exceed
+ * that size is refused with HRN_E_BADPARAM.  Every call on a GPU uses that GPU's one workspace: calls that overlap
+ * in time on one GPU (different streams or threads) race; nothing in it needs to be zero between calls.  Calls no
+ * hipMalloc / hipFree.
+ */
+#define HRN_STATIC_WORKSPACE_BYTES (32u << 20)
+int hrn_launch_splitk_static(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
+
 /* `count` back-to-back launches of the same problem from one host call (the inner loop of a time_evaluator
  * repeat, runner/measure_methods.py:138-145, without the events). */
 int hrn_launch_repeat(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C,
