@@ -226,7 +226,12 @@ ADAPTERS = {
 }
 
 
-def run_operator(mod, info, inputs, group_m=8):
+# adapters whose ACTIVATION operand passes through unchanged when its channel count is a whole 16-byte chunk: the
+# caller's tensor is already channels-last, only the (constant) filter is reordered once
+ACTIVATION_AS_IS = ('identity', 'c1d_nwc', 'c2d_hwio')
+
+
+def run_operator(mod, info, inputs, group_m=8, split_k=0):
     """Runs one operator of the registry on device tensors given in the reference's own layouts.
 
     ``info`` is the dictionary the operator definition handed to ``ctx.set_info``; ``mod`` an instance of the
@@ -236,7 +241,7 @@ def run_operator(mod, info, inputs, group_m=8):
     if info['operator'] == 'conv2d_nhwc':
         c = info['conv']
         C = conv2d_nhwc(mod, A, Bm, (c['stride'], c['stride_w']), (c['pad'], c['pad_w']), (c['dil'], c['dil_w']),
-                        group_m=group_m)
+                        group_m=group_m, split_k=split_k)
     else:
-        C = gemm(mod, A, Bm, group_m=group_m)
+        C = gemm(mod, A, Bm, group_m=group_m, split_k=split_k)
     return fin(info, C)

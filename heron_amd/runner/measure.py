@@ -30,7 +30,10 @@ class MeasureErrorNo(object):
     VERIFY_FAILED = 100
 
 
-BuildResult = namedtuple("BuildResult", ["desc_tuple", "problem", "arg_info", "error", "time_cost"])
+# ``adapter``: the operator's info dictionary when its operands go through an operand adapter (then the pre-stage is
+# part of what gets timed), None for operators that hand their tensors to the kernel as they are
+BuildResult = namedtuple("BuildResult", ["desc_tuple", "problem", "arg_info", "error", "time_cost", "adapter"],
+                         defaults=(None,))
 
 
 def measure_option(builder, runner):

@@ -222,7 +222,14 @@ class KnobManager:
             candidates = self.get_knob_candidates(key)
             hint[key] = candidates[random.randint(0, len(candidates) - 1)]
         valid, point = self.solver.solve(hint=hint, known=known, bounds=bounds)
-        assert valid
+        for _ in range(3):
+            if valid or self.solver.last_status != 'unknown':
+                break
+            # the randomised search gave up, which proves nothing: try again from other hints
+            hint = {k: random.choice(self.get_knob_candidates(k)) for k in hint}
+            valid, point = self.solver.solve(hint=hint, known=known, bounds=bounds)
+        if not valid:
+            raise RuntimeError("no feasible point (%s)" % self.solver.last_status)
         self._valid = valid
         self._store(point)
         return valid, point

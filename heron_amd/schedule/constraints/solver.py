@@ -186,6 +186,9 @@ class Solver:
         self.primitives = []
         self.fail_budget = 400
         self.restarts = 8
+        self.last_status = None         # 'feasible' | 'infeasible' | 'unknown' of the last solve
+        self.budget_hits = 0            # searches given up on their fail budget since construction
+        self._budget_hit = False
 
     def addVal(self, name, low, up, def_val):
         assert name not in self.vals.keys()
@@ -287,19 +290,37 @@ class Solver:
                     break
                 fails += 1
                 if fails > self.fail_budget:
+                    self._budget_hit = True
                     return None
             if not advanced:
                 return None
 
     def _solve(self, hint, known, bounds, fixed=None, rng=None):
+        """(valid, point).  ``self.last_status`` says which kind of "not valid" it was: 'infeasible' (propagation or an
+        exhausted search proved that no point exists) or 'unknown' (every restart ran out of its fail budget; the
+        system may still be feasible - the reference's CP-SAT is complete and never reports this)."""
         rng = rng or random
+        self.last_status = 'infeasible'
         root = self._root(known, bounds, fixed)
         if root is None:
             return False, None
-        for _ in range(self.restarts):
-            res = self._search(root, hint, rng)
-            if res is not None:
-                return True, res
+        budget = self.fail_budget
+        try:
+            for attempt in range(self.restarts + 1):
+                if attempt == self.restarts:
+                    # last resort: one search with a budget large enough to settle most systems either way
+                    self.fail_budget = budget * 25
+                self._budget_hit = False
+                res = self._search(root, hint, rng)
+                if res is not None:
+                    self.last_status = 'feasible'
+                    return True, res
+                if not self._budget_hit:
+                    return False, None          # the search space was exhausted: proven infeasible
+                self.budget_hits += 1
+        finally:
+            self.fail_budget = budget
+        self.last_status = 'unknown'
         return False, None
 
     # ------------------------------------------------------------------ reference interface

@@ -34,6 +34,7 @@ def main():
     parser.add_argument("-m", "--max-trials", type=int, default=int(1e6))
     parser.add_argument("-o", "--out", default="", help="write the per-layer table as JSON")
     parser.add_argument("-v", "--verbose", action="store_true")
+    parser.add_argument("--check", action="store_true", help="verify every measured kernel against a host reference")
     args = parser.parse_args()
 
     config = makeConfig(args)
@@ -54,7 +55,7 @@ def main():
                 config.tuned = rec
         print(keys[i], op_name, case, flush=True)
         env = Env(option, config)
-        latency = run(op_name, keys[i], case + [config.in_dtype, config.out_dtype], env, runner)
+        latency = run(op_name, keys[i], case + [config.in_dtype, config.out_dtype], env, runner, args.check)
         rows.append(dict(case=keys[i], op=op_name, shape=case, times=times, latency_ms=latency))
     plain = weighted = 0.0
     for r in rows:

@@ -73,9 +73,9 @@ def make_env(tmp_path, method="CGA", trials=48, case=("gemm", [1024, 1024, 1024]
     cfg.codegen_type, cfg.target_name, cfg.get_op = 'GPU_MFMA', 'rocm', getOpFromName
     cfg.out_name = str(tmp_path / "OPS")
     cfg.feasible_file_path = str(tmp_path / "feasible.json")
-    cfg.feasible_samples = 96
+    cfg.feasible_samples = 48
     cfg.opt_method, cfg.max_trials = method, trials
-    cfg.measure_time_per_round, cfg.pop_num, cfg.select_num, cfg.iter_walks = 16, 24, 12, 2
+    cfg.measure_time_per_round, cfg.pop_num, cfg.select_num, cfg.iter_walks = 16, 16, 8, 1
     cfg.parallel_num, cfg.history_topk = 2, 8
     cfg.in_dtype, cfg.out_dtype = dtype, dtype
     env = Env(measure_option(FakeBuilder(), FakeRunner()), cfg)
