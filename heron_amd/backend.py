@@ -142,6 +142,7 @@ SYMBOLS = {
     "hrn_problem_conv2d_hw": (None, [ctypes.POINTER(Problem)] + [_i] * 13),
     "hrn_probe_mfma": (_i, [_i, _i, _i, ctypes.POINTER(_d), _vp]),
     "hrn_probe_copy": (_i, [_vp, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
+    "hrn_probe_launch": (_i, [_i, _i, ctypes.POINTER(_d), _vp]),
     "hrn_last_error": (ctypes.c_char_p, []),
     "hrn_version": (ctypes.c_char_p, []),
 }
@@ -228,6 +229,13 @@ def probe_mfma(dtype, mfma=32, random_operands=True, stream=0):
     """Dense T(FL)OP/s of a register-resident MFMA loop on all CUs (measured roofline denominator)."""
     out = _d()
     _check(lib().hrn_probe_mfma(dtype, mfma, 1 if random_operands else 0, ctypes.byref(out), stream))
+    return out.value
+
+
+def probe_launch(grid=256, repeat=2000, stream=0):
+    """Microseconds per back-to-back dispatch of a kernel that does nothing."""
+    out = ctypes.c_double()
+    _check(lib().hrn_probe_launch(grid, repeat, ctypes.byref(out), stream))
     return out.value
 
 

@@ -622,9 +622,32 @@ __global__ void __launch_bounds__(256) probe_copy_kernel(const pv4i* __restrict_
     for (; i < n16; i += stride) dst[i] = src[i];
 }
 
+// does nothing: what the device needs to start and retire one dispatch of `grid` workgroups
+__global__ void __launch_bounds__(256) probe_empty_kernel(int* sink) {
+    if (sink && threadIdx.x == 0x7fffffff) *sink = 0;
+}
+
 }  // namespace
 
 extern "C" {
+
+int hrn_probe_launch(int grid, int repeat, double* us_out, void* stream) {
+    if (!us_out || grid < 1 || grid > (1 << 20) || repeat < 1) return fail(HRN_E_BADPARAM, "probe arguments");
+    hipStream_t st = (hipStream_t)stream;
+    EventPair ev;
+    HIP_TRY(ev.create());
+    hipEvent_t e0 = ev.e0, e1 = ev.e1;
+    for (int i = 0; i < 20; ++i) probe_empty_kernel<<<grid, 256, 0, st>>>(nullptr);
+    (void)hipEventRecord(e0, st);
+    for (int i = 0; i < repeat; ++i) probe_empty_kernel<<<grid, 256, 0, st>>>(nullptr);
+    (void)hipEventRecord(e1, st);
+    hipError_t e = hipEventSynchronize(e1);
+    float ms = 0;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    if (e != hipSuccess) return fail(HRN_E_LAUNCH, "probe: %s", hipGetErrorString(e));
+    *us_out = ms * 1e3 / repeat;
+    return HRN_OK;
+}
 
 int hrn_probe_mfma(int dtype, int mfma, int random_operands, double* tops_out, void* stream) {
     if (!tops_out || (mfma != 32 && mfma != 16) || (dtype != HRN_DT_F16 && dtype != HRN_DT_U8S8))

@@ -64,6 +64,11 @@ constexpr int EPI = HRN_EPI;
 #define HRN_ABLATE 0
 #endif
 constexpr int ABL = HRN_ABLATE;
+// timing study only (results are wrong): keep HRN_FAKE_DEPTH k-tiles in flight, written round-robin over the NS stages
+#ifndef HRN_FAKE_DEPTH
+#define HRN_FAKE_DEPTH 0
+#endif
+constexpr int FD = HRN_FAKE_DEPTH;
 // Conv window mode (HRN_OP=1, stride 1, dilation 1, 'same' padding): instead of fetching an im2col tile of A for every
 // filter tap, the workgroup loads ONCE the window of input pixels its BM output pixels can reach (a contiguous range
 // of BM + 2*(pad_h*W + pad_w) pixels, all channels) and every tap reads its operand fragments from that window at a row offset
@@ -146,7 +151,7 @@ static_assert(!SPLITK || !CW, "split-K uses the im2col load path");
 static_assert(LDS_BYTES <= 163840, "LDS");
 static_assert(EPI == 0 || (MT * (SW * OES / 16)) % 64 == 0, "staged epilogue: a strip must split into whole wave stores");
 static_assert(SWZ == 0 || (CPR << (SWZ - 1)) <= MT, "swizzle period must fit in one MFMA tile");
-static_assert((NS - 1) * LPT <= 63, "vmcnt range");
+static_assert(((FD ? FD : NS) - 1) * LPT <= 63, "vmcnt range");
 static_assert(NT <= 1024, "threads");
 static_assert(DT == 0 || NS * STAGE_BYTES >= WM * BN * 4, "column sums must fit the stages");
 
@@ -672,8 +677,8 @@ hrn_mfma_kernel(const HrnKArgs a) {
 
     // ---- prologue: fill all stages, wait for tile 0 ----
 #pragma unroll
-    for (int s = 0; s < NS; ++s) issue_tile(s);
-    wait_and_barrier<(NS - 1) * LPT, 0>();
+    for (int s = 0; s < (FD ? FD : NS); ++s) issue_tile(s % NS);
+    wait_and_barrier<((FD ? FD : NS) - 1) * LPT, 0>();
     read_frags(0, 0, 0);
 
     int stage = 0;
@@ -746,9 +751,9 @@ hrn_mfma_kernel(const HrnKArgs a) {
                     if (stores_between && kt <= NS - 2) wait_and_barrier<(NS - 2) * LPT + STORES_PER_TILE, 0>();
                     else wait_and_barrier<(NS - 2) * LPT, 0>();
                 } else if constexpr (ABL & 4) {
-                    wait_only<(NS - 2) * LPT, 0>();
+                    wait_only<((FD ? FD : NS) - 2) * LPT, 0>();
                 } else {
-                    wait_and_barrier<(NS - 2) * LPT, 0>();
+                    wait_and_barrier<((FD ? FD : NS) - 2) * LPT, 0>();
                 }
                 const bool rag = begin_issue();
                 conv_tap();

@@ -71,9 +71,7 @@ def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8, split_k
 def _pad_last(t, to):
     if t.shape[-1] == to:
         return t.contiguous()
-    out = torch.zeros(t.shape[:-1] + (to,), dtype=t.dtype, device=t.device)
-    out[..., :t.shape[-1]] = t
-    return out
+    return torch.nn.functional.pad(t, (0, to - t.shape[-1])).contiguous()      # one pass
 
 
 def _prep_identity(info, A, Bm):
@@ -128,6 +126,10 @@ def _prep_c1d_ncw(info, X, F):            # (N,CI,W), (CO,CI,KW)
 
 def _prep_c2d_nchw(info, X, F):           # (N,CI,H,W), (CO,CI,KH,KW)
     return _pad_last(X.permute(0, 2, 3, 1), _cpad(info)), _pad_last(F.permute(0, 2, 3, 1), _cpad(info))
+
+
+def _prep_c2d_krsc(info, X, F):           # (N,H,W,CI), (CO,KH,KW,CI) with CI short of a whole 16-byte chunk
+    return _pad_last(X, _cpad(info)), _pad_last(F, _cpad(info))
 
 
 def _prep_c2d_hwio(info, X, F):           # (N,H,W,CI), (KH,KW,CI,CO)
@@ -219,6 +221,7 @@ ADAPTERS = {
     'c1d_ncw': (_prep_c1d_ncw, _fin_c1d_ncw),
     'c2d_nchw': (_prep_c2d_nchw, _fin_nchw),
     'c2d_hwio': (_prep_c2d_hwio, _fin_identity),
+    'c2d_krsc': (_prep_c2d_krsc, _fin_identity),
     'c3d_ndhwc': (_prep_c3d_ndhwc, _fin_c3d_ndhwc),
     'c3d_ncdhw': (_prep_c3d_ncdhw, _fin_c3d_ncdhw),
     't2d_nchw': (_prep_t2d_nchw, _fin_nchw),
@@ -228,7 +231,7 @@ ADAPTERS = {
 
 # adapters whose ACTIVATION operand passes through unchanged when its channel count is a whole 16-byte chunk: the
 # caller's tensor is already channels-last, only the (constant) filter is reordered once
-ACTIVATION_AS_IS = ('identity', 'c1d_nwc', 'c2d_hwio')
+ACTIVATION_AS_IS = ('identity', 'c1d_nwc', 'c2d_hwio', 'c2d_krsc')
 
 
 def run_operator(mod, info, inputs, group_m=8, split_k=0):

@@ -44,8 +44,13 @@ def heron_conv2d_nhwc(ctx, N, H, W, CI, CO, KH, KW, stride, padding, dilation, *
     kind = element_kind(in_dtype)
     if w_format is not None and kind != "u8s8":
         raise ValueError("w_format belongs to the quantized operator")
-    if kind == "f16" and CI % 8 or kind == "u8s8" and CI % 16:
-        raise ValueError("CI must cover whole 16-byte channel chunks (multiple of 8 for fp16, 16 for uint8)")
+    chunk = 8 if kind == "f16" else 16
+    extra = {}
+    if CI % chunk:
+        # fewer channels than a whole 16-byte chunk (the 3-channel stem of the vision networks): the kernel runs on
+        # zero-padded channels, the 'c2d_krsc' adapter pads activation and filter, the result needs no reorder
+        extra = {'adapter': 'c2d_krsc', 'reference_args': dict(input=(N, H, W, CI), filter=(CO, KH, KW, CI)), 'ci': CI}
+        CI = (CI + chunk - 1) // chunk * chunk
     HO = conv_out_size(H, KH, sh, ph, dh)
     WO = conv_out_size(W, KW, sw, pw, dw)
     a_dt, b_dt, o_dt = ("float16", "float16", "float16") if kind == "f16" else ("uint8", "int8", "int32")
@@ -55,7 +60,7 @@ def heron_conv2d_nhwc(ctx, N, H, W, CI, CO, KH, KW, stride, padding, dilation, *
     conv = dict(w_format=w_format, N=N, H=H, W=W, CI=CI, CO=CO, KH=KH, KW=KW, stride=sh, pad=ph, dil=dh, stride_w=sw, pad_w=pw, dil_w=dw,
                 HO=HO, WO=WO)
     ctx.set_info(mfma_info(kind, out.op.name, Input.name, Filter.name,
-                           dict(batch=1, M=N * HO * WO, N=CO, K=KH * KW * CI), 'conv2d_nhwc', {'conv': conv}))
+                           dict(batch=1, M=N * HO * WO, N=CO, K=KH * KW * CI), 'conv2d_nhwc', dict(extra, conv=conv)))
     ctx.set_axis_map({
         'input.lds': ['s_0', 's_1', 's_2', 'r_0', 'r_1', 'r_2'],
         'filter.lds': ['s_3', 'r_0', 'r_1', 'r_2'],

@@ -189,6 +189,7 @@ class Solver:
         self.last_status = None         # 'feasible' | 'infeasible' | 'unknown' of the last solve
         self.budget_hits = 0            # searches given up on their fail budget since construction
         self._budget_hit = False
+        self._sampled_out = False
 
     def addVal(self, name, low, up, def_val):
         assert name not in self.vals.keys()
@@ -264,6 +265,13 @@ class Solver:
         others = [k for k in names if k not in hint]
         rng.shuffle(hinted)
         rng.shuffle(others)
+        # variables with an enumerated domain before interval variables, and among them the many-valued ones (the
+        # knobs) before the two-valued ones (their one-hot companions): propagation fixes most of the rest once the
+        # knobs are chosen
+        def rank(k):
+            d = root.doms[k]
+            return 2 if d.vals is None else (1 if len(d.vals) <= 2 else 0)
+        others.sort(key=rank)
         order = hinted + others
         fails = 0
         # explicit stack of (store, position in order, remaining values)
@@ -280,6 +288,9 @@ class Solver:
             while stack:
                 S0, pos0, cands = stack[-1]
                 if not cands:
+                    d0 = S0.doms[order[pos0]]
+                    if d0.vals is None and d0.hi - d0.lo + 1 > 8:
+                        self._sampled_out = True        # an interval was only sampled: nothing is proven
                     stack.pop()
                     continue
                 v = cands.pop(0)
@@ -310,12 +321,12 @@ class Solver:
                 if attempt == self.restarts:
                     # last resort: one search with a budget large enough to settle most systems either way
                     self.fail_budget = budget * 25
-                self._budget_hit = False
+                self._budget_hit = self._sampled_out = False
                 res = self._search(root, hint, rng)
                 if res is not None:
                     self.last_status = 'feasible'
                     return True, res
-                if not self._budget_hit:
+                if not self._budget_hit and not self._sampled_out:
                     return False, None          # the search space was exhausted: proven infeasible
                 self.budget_hits += 1
         finally:

@@ -50,10 +50,15 @@ class Task:
         self.sched_desc = ctx.sched_desc
         self.template_info = ctx.tensorize_info
         self.knob_manager.is_building = False
-        feasible, _ = self.knob_manager.solver.solve({}, {})
+        solver = self.knob_manager.solver
+        feasible, _ = solver.solve({}, {})
+        for _ in range(4):
+            if feasible or solver.last_status != 'unknown':
+                break
+            feasible, _ = solver.solve({}, {})      # the randomised search gave up; that proves nothing
         self.dump_constraints()
         if not feasible:
-            raise AssertionError("the template has no feasible instance for this shape")
+            raise AssertionError("the template has no feasible instance for this shape (solver: %s)" % solver.last_status)
 
     def dump_constraints(self):
         log_dir = getattr(self.config, "log_dir", None)

@@ -26,6 +26,9 @@ class Tuner:
         self.total_sample_time = 0
         self.total_measure_time = 0
         self.feasible = None
+        # share of the measuring rounds, at the end of a run, whose candidates are the one-knob neighbours of the best
+        # measured points (constrained tuners switch it on); the reference has no such phase
+        self.refine_share = 0.0
 
     def buildCostModel(self, task):
         self.cost_model = XGBoostCostModel(task, self.config)
@@ -84,7 +87,15 @@ class Tuner:
             measure_s = time.time()
             # points known to violate the constraint system are not worth a build (the reference selects among them
             # too and lets the build fail, tuner.py:66-70)
-            pop = self.epsilon_select(env, [x for x in all_pop if x.valid], 0.6, select_num)
+            measuring_rounds = total_iters - (1 if last_iter_select_num == 0 else 0)
+            refine_rounds = int(self.refine_share * measuring_rounds + 0.5) if measuring_rounds >= 3 else 0
+            if do_measure and select_num > 0 and iter_no >= measuring_rounds - refine_rounds:
+                near = self.greedy_select(env, self.incumbent_neighbours(env), select_num)
+                print("refinement round: %d unmeasured one-knob neighbours of the best points" % len(near))
+                rest = [x for x in all_pop if x.valid and x.stmt_code not in {n.stmt_code for n in near}]
+                pop = near + self.epsilon_select(env, rest, 0.6, select_num - len(near)) if len(near) < select_num else near
+            else:
+                pop = self.epsilon_select(env, [x for x in all_pop if x.valid], 0.6, select_num)
             if do_measure and pop != []:
                 samples = self.FilterSamples(pop, env)
                 self.measure(samples, env)
@@ -216,6 +227,31 @@ class Tuner:
             sample.violation = 0.0
             ret.append(sample)
         return ret
+
+    def incumbent_neighbours(self, env, top=3):
+        """Feasible points that differ from one of the ``top`` best measured points in exactly one knob (the solver
+        re-derives the dependent variables), scored by the cost model."""
+        out, seen = [], set()
+        for base in reversed(self.history_topk_samples(env, top)):
+            geno = base.knob_manager.solved_knob_vals_genotype
+            names = base.knob_manager.knob_names
+            for name in names:
+                for cand in base.knob_manager.get_knob_candidates(name):
+                    if cand == geno[name]:
+                        continue
+                    s = Sample(env.task)
+                    point, valid = s.knob_manager.validate({n: (cand if n == name else geno[n]) for n in names})
+                    if not valid:
+                        continue
+                    s.point, s.valid, s.stmt_code = point, True, Code(point)
+                    if s.stmt_code in seen:
+                        continue
+                    seen.add(s.stmt_code)
+                    out.append(s)
+        perfs = self.predict(out) if out else []
+        for s, p in zip(out, perfs):
+            s.predict, s.violation = p, 0
+        return out
 
     def repredict(self, pop):
         for sample in pop:

@@ -225,7 +225,10 @@ int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, co
  * clock); hrn_probe_copy times a 16-byte-per-lane
  * copy kernel over `bytes` of caller-owned device memory and returns GB/s counting read + write.
  * The copy kernel is also the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters.
+ * hrn_probe_launch times `repeat` back-to-back dispatches of a kernel that does nothing (`grid` workgroups of 256
+ * lanes) and returns microseconds per dispatch: the floor under every small layer's latency.
  */
+int hrn_probe_launch(int grid, int repeat, double* us_out, void* stream);
 int hrn_probe_mfma(int dtype, int mfma, int random_operands, double* tops_out, void* stream);
 int hrn_probe_copy(const void* src, void* dst, size_t bytes, int repeat, double* gbs_out, void* stream);
 

@@ -2,8 +2,8 @@
 network experiment tunes (tests/figure10/configs/*.json, read here as JSON data), re-targeted at the rocm registry.
 
 Layers keep the reference's ``[op, shape, count]`` form.  ``c2d`` entries run on the NHWC operator (activations stay
-NHWC between layers on this backend); a layer whose channel count is not a whole 16-byte chunk (the 3-channel stem)
-is routed to ``c2d_nchw``, whose operand adapter pads the channels.  ``max_trials`` is cut to what one GPU session
+NHWC between layers on this backend); for a layer whose channel count is not a whole 16-byte chunk (the 3-channel stem)
+that operator pads the channels through its operand adapter, and the timing includes the padding pass.  ``max_trials`` is cut to what one GPU session
 affords; pass ``-m`` to the runner to change it.
 
 usage: python make_configs.py /path/to/reference/tests/figure10/configs
@@ -19,8 +19,6 @@ def convert(src, max_trials=256):
     c = json.load(open(src))["config"]
     cases = {}
     for key, (op, shape, count) in c["cases"].items():
-        if op == "c2d" and shape[3] % 8:
-            op = "c2d_nchw"
         cases[key.strip()] = [op, shape, count]
     out = dict(c)
     out["cases"] = cases

@@ -145,3 +145,32 @@ def test_knob_manager_builders_and_operators():
     assert valid and child.solver.SATScore(child.solved_knob_vals_phenotype) == 0
     _, ok = child.validate({"P#x": 8, "P#y": 8})
     assert not ok                                               # 64 > 32 and x == y
+
+
+def test_status_distinguishes_proven_from_given_up():
+    """'infeasible' is only claimed when propagation or an exhaustive search proves it; a search that merely sampled
+    a wide interval, or ran out of its fail budget, reports 'unknown'."""
+    s = Solver()
+    s.addVal("x", 0, 3, 0)
+    s.addVal("y", 0, 3, 0)
+    s.primitives.append(LT(["x", "y"]))
+    s.primitives.append(LT(["y", "x"]))
+    ok, _ = s.solve({}, {})
+    assert not ok and s.last_status == 'infeasible'
+    # one feasible value in a wide interval that propagation cannot single out (x*x == y*y + 2001 has the integer
+    # solutions x = 1001, y = 1000 only... the solver either finds it or must say that it does not know)
+    t = Solver()
+    t.addVal("x", 0, 5000, 0)
+    t.addVal("y", 0, 5000, 0)
+    t.addVal("xx", 0, 25000000, 0)
+    t.addVal("yy", 0, 25000000, 0)
+    t.primitives.append(ProdTwo(["xx", ["x", "x"]]))
+    t.primitives.append(ProdTwo(["yy", ["y", "y"]]))
+    t.primitives.append(Sum(["xx", ["yy", 2001]]))
+    t.fail_budget, t.restarts = 20, 2
+    random.seed(5)
+    ok, point = t.solve({}, {})
+    if ok:
+        assert point[0] == 1001 and point[1] == 1000
+    else:
+        assert t.last_status == 'unknown'

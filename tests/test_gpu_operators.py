@@ -120,6 +120,13 @@ def test_conv2d_nchw_dilated_and_transposed(dtype, hrn):
         print("c2d_nchw", dtype, (N, H, W, CI, CO, KH, KW, s, p, d), flush=True)
         info, _ = declare("c2d_nchw", [N, H, W, CI, CO, KH, KW, s, p, d], dtype)
         check(hostops.run_operator(module(info), info, [dev(X), dev(F)]), oracle.conv2d_nchw_ref(X, F, s, p, d), f16)
+    # channels-last conv whose channel count is short of a 16-byte chunk: padded by the adapter, result as it is
+    for (N, H, W, CI, CO, KH, KW, s, p, d) in [(2, 20, 20, 3, 16, 7, 7, 2, 3, 1), (1, 9, 11, 20, 8, 3, 3, 1, 1, 1)]:
+        X, F = rnd((N, H, W, CI), 15, a_dt), rnd((CO, KH, KW, CI), 16, b_dt)
+        print("c2d short channels", dtype, (N, H, W, CI, CO, KH, KW, s, p, d), flush=True)
+        info, _ = declare("c2d", [N, H, W, CI, CO, KH, KW, s, p, d], dtype)
+        ref = oracle.conv2d_nhwc_f32(X, F, s, p, d) if f16 else oracle.conv2d_nhwc_u8s8s32(X, F, s, p, d)
+        check(hostops.run_operator(module(info), info, [dev(X), dev(F)]), ref, f16)
     for (N, H, W, CI, CO, KH, KW, s, p, d) in [(2, 20, 20, 16, 16, 3, 3, 1, 2, 2), (1, 17, 13, 8, 12, 3, 3, 2, 3, 3)]:
         X, F = rnd((N, H, W, CI), 9, a_dt), rnd((KH, KW, CI, CO), 10, b_dt)
         print("dil", dtype, (N, H, W, CI, CO, KH, KW, s, p, d), flush=True)

@@ -74,6 +74,9 @@ def test_conv2d_variants():
           oracle.conv2d_nchw_ref(X, F, (2, 1), (1, 2), 1))
     X, F = rnd((1, 17, 13, 8), 10), rnd((3, 3, 8, 12), 11)
     close(through_adapter("dil", [1, 17, 13, 8, 12, 3, 3, 2, 3, 3], [X, F]), oracle.dil_nhwc_ref(X, F, 2, 3, 3))
+    # channels-last conv with 3 input channels (the stem of the vision networks): padded to a whole chunk, no reorder
+    X, F = rnd((2, 20, 20, 3), 16), rnd((16, 7, 7, 3), 17)
+    close(through_adapter("c2d", [2, 20, 20, 3, 16, 7, 7, 2, 3, 1], [X, F]), oracle.conv2d_nhwc_f32(X, F, 2, 3, 1))
 
 
 @pytest.mark.parametrize("s,p,d,op", [(2, 1, 1, 0), (2, 1, 1, 1), (1, 0, 1, 0), (3, 2, 2, 1)])
