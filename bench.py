@@ -161,6 +161,7 @@ def run_probes(torch, B):
         "mfma_i8_const_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 32, False, st),
         "mfma_i8_random_operands_TOPs": B.probe_mfma(B.HRN_DT_U8S8, 32, True, st),
         "hbm_copy_1GiB_read_plus_write_GBs": B.probe_copy(src.data_ptr(), dst.data_ptr(), n, 10, st),
+        "hbm_read_1GiB_GBs": B.probe_read(src.data_ptr(), n, 10, st),
         "empty_kernel_256wg_us_per_launch": B.probe_launch(256, 2000, st),
         "empty_kernel_2048wg_us_per_launch": B.probe_launch(2048, 2000, st),
     }

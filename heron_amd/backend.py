@@ -143,6 +143,7 @@ SYMBOLS = {
     "hrn_probe_mfma": (_i, [_i, _i, _i, ctypes.POINTER(_d), _vp]),
     "hrn_probe_copy": (_i, [_vp, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_probe_launch": (_i, [_i, _i, ctypes.POINTER(_d), _vp]),
+    "hrn_probe_read": (_i, [_vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_last_error": (ctypes.c_char_p, []),
     "hrn_version": (ctypes.c_char_p, []),
 }
@@ -236,6 +237,13 @@ def probe_launch(grid=256, repeat=2000, stream=0):
     """Microseconds per back-to-back dispatch of a kernel that does nothing."""
     out = ctypes.c_double()
     _check(lib().hrn_probe_launch(grid, repeat, ctypes.byref(out), stream))
+    return out.value
+
+
+def probe_read(src_ptr, nbytes, repeat=10, stream=0):
+    """GB/s of a read-only stream over device memory."""
+    out = ctypes.c_double()
+    _check(lib().hrn_probe_read(src_ptr, nbytes, repeat, ctypes.byref(out), stream))
     return out.value
 
 

@@ -622,6 +622,20 @@ __global__ void __launch_bounds__(256) probe_copy_kernel(const pv4i* __restrict_
     for (; i < n16; i += stride) dst[i] = src[i];
 }
 
+// streams `n16` 16-byte words through every lane without storing anything: the read-only counterpart of the copy probe
+__global__ void __launch_bounds__(256) probe_read_kernel(const pv4i* __restrict__ src, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    pv4i acc = {0, 0, 0, 0};
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        const pv4i v0 = src[i], v1 = src[i + stride], v2 = src[i + 2 * stride], v3 = src[i + 3 * stride];
+        acc |= v0 | v1 | v2 | v3;
+    }
+    for (; i < n16; i += stride) acc |= src[i];
+    const int keep = acc.x | acc.y | acc.z | acc.w;
+    asm volatile("" ::"v"(keep));   // keeps the loads live; nothing is stored
+}
+
 // does nothing: what the device needs to start and retire one dispatch of `grid` workgroups
 __global__ void __launch_bounds__(256) probe_empty_kernel(int* sink) {
     if (sink && threadIdx.x == 0x7fffffff) *sink = 0;
@@ -630,6 +644,29 @@ __global__ void __launch_bounds__(256) probe_empty_kernel(int* sink) {
 }  // namespace
 
 extern "C" {
+
+int hrn_probe_read(const void* src, size_t bytes, int repeat, double* gbs_out, void* stream) {
+    if (!src || !gbs_out || bytes < 16 || bytes % 16 || repeat < 1) return fail(HRN_E_BADPARAM, "probe arguments");
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t pr;
+    HIP_TRY(hipGetDeviceProperties(&pr, dev));
+    hipStream_t st = (hipStream_t)stream;
+    EventPair ev;
+    HIP_TRY(ev.create());
+    hipEvent_t e0 = ev.e0, e1 = ev.e1;
+    const int grid = pr.multiProcessorCount * 16;
+    probe_read_kernel<<<grid, 256, 0, st>>>((const pv4i*)src, bytes / 16);
+    (void)hipEventRecord(e0, st);
+    for (int i = 0; i < repeat; ++i) probe_read_kernel<<<grid, 256, 0, st>>>((const pv4i*)src, bytes / 16);
+    (void)hipEventRecord(e1, st);
+    hipError_t e = hipEventSynchronize(e1);
+    float ms = 0;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    if (e != hipSuccess) return fail(HRN_E_LAUNCH, "probe: %s", hipGetErrorString(e));
+    *gbs_out = (double)bytes * repeat / (ms * 1e-3) / 1e9;
+    return HRN_OK;
+}
 
 int hrn_probe_launch(int grid, int repeat, double* us_out, void* stream) {
     if (!us_out || grid < 1 || grid > (1 << 20) || repeat < 1) return fail(HRN_E_BADPARAM, "probe arguments");

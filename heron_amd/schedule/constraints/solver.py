@@ -265,13 +265,6 @@ class Solver:
         others = [k for k in names if k not in hint]
         rng.shuffle(hinted)
         rng.shuffle(others)
-        # variables with an enumerated domain before interval variables, and among them the many-valued ones (the
-        # knobs) before the two-valued ones (their one-hot companions): propagation fixes most of the rest once the
-        # knobs are chosen
-        def rank(k):
-            d = root.doms[k]
-            return 2 if d.vals is None else (1 if len(d.vals) <= 2 else 0)
-        others.sort(key=rank)
         order = hinted + others
         fails = 0
         # explicit stack of (store, position in order, remaining values)

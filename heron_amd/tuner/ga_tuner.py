@@ -72,7 +72,7 @@ class CGATuner(GATuner):
         super().__init__(config)
         # the last quarter of the measuring rounds refines the incumbents knob by knob: the fine knobs (issue order,
         # load spread, raster group, epilogue kind) move a good tile by a few percent, less than the cost model resolves
-        self.refine_share = 0.25
+        self.refine_share = float(getattr(config, 'refine_share', 0.25))
 
     def check_feasible_exits(self, env, num=1e3):
         return

@@ -229,6 +229,9 @@ int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, co
  * lanes) and returns microseconds per dispatch: the floor under every small layer's latency.
  */
 int hrn_probe_launch(int grid, int repeat, double* us_out, void* stream);
+/* hrn_probe_read streams `bytes` of caller-owned device memory through the lanes without storing (GB/s read): what
+ * a kernel that only reads, like the P x V batch_matmul, can draw from HBM when the buffer exceeds the caches. */
+int hrn_probe_read(const void* src, size_t bytes, int repeat, double* gbs_out, void* stream);
 int hrn_probe_mfma(int dtype, int mfma, int random_operands, double* tops_out, void* stream);
 int hrn_probe_copy(const void* src, void* dst, size_t bytes, int repeat, double* gbs_out, void* stream);
 

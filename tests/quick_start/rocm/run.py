@@ -83,7 +83,7 @@ def run(op_name, task_name, params, env, runner, check=False):
     s, args = task.apply_best(config.tuned)
     print("Best instance:", s.describe())
     latency = runner.time_instance(s, args, number=config.runner_number, repeat=config.runner_repeat,
-                                   min_repeat_ms=500) * 1e3
+                                   min_repeat_ms=500, cold=getattr(config, "cold", False)) * 1e3
     if latency > 0:
         print("PASS")
     return latency
@@ -103,6 +103,9 @@ if __name__ == '__main__':
     parser.add_argument("-v", "--verbose", action="store_true", help="Show some information if enabled.")
     parser.add_argument("-m", "--max-trials", type=int, default=int(1e6), help="Max trials by command line")
     parser.add_argument("--check", action="store_true", help="verify measured kernels against a host reference")
+    parser.add_argument("--cold", action="store_true",
+                        help="time every launch from flushed caches (the runner's enable_cpu_cache_flush of "
+                             "tests/quick_start/dlboost/run.py:89-96, on the GPU): for cases bound by HBM traffic")
     parser.add_argument("--pretrained", type=str, default="",
                         help="comma separated records.txt files of earlier tasks of the same operator: steer the search "
                              "with a cost model fitted on them instead of training one from scratch")
@@ -115,8 +118,10 @@ if __name__ == '__main__':
     config.tuned = args.tuned
     config.verbose = args.verbose
     config.pretrained_records = [p for p in args.pretrained.split(",") if p]
+    config.cold = args.cold
     runner = HeronRunner.LocalRunner(number=config.runner_number, repeat=config.runner_repeat, min_repeat_ms=0,
-                                     timeout=config.runner_timeout, device_id=args.device_id)
+                                     timeout=config.runner_timeout, enable_cpu_cache_flush=args.cold,
+                                     device_id=args.device_id)
     measure_option = HeronRunner.measure_option(
         builder=HeronRunner.LocalBuilder(timeout=config.build_timeout),
         runner=runner,
