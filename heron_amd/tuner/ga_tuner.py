@@ -1,9 +1,15 @@
-"""Genetic tuners (tuner/ga_tuner.py:13-110 of the reference).
+"""Genetic tuners (the family of tuner/ga_tuner.py:13-166 of the reference).
 
-CGATuner is the constrained genetic algorithm: each walk draws a random 20 % of *all* CSP variables
-as key variables, roulette-selects parents, and creates every child by solving the CSP with each key
-variable restricted to one of its two parents' values (one key left free as the mutation), so every
-child is feasible by construction.
+All of them share one generation step: pick the key variables, order and select parents, breed ``pop_num`` children,
+score them, keep the 20 best seen so far in the breeding pool.  The tuners differ in how a child is made from two
+parents (``BREED``) and in how parents are ranked and selected:
+
+* ``GA``    one-point crossover + one mutated knob, validated afterwards (children may be infeasible);
+* ``CGA``   constrained: a random 20 % of *all* CSP variables are key variables, and a child is the solver's answer to
+            "each key variable equals one of its two parents' values, one key left free" - feasible by construction;
+* ``RCGA``  CGA with fresh key variables for every breeding call;
+* ``SRGA``  unconstrained operators over all variables, stochastic ranking against the violation;
+* ``SDGA``  the crossed genotype is repaired into a feasible phenotype by the solver (SAT decoding).
 """
 import os
 import random
@@ -15,27 +21,94 @@ from ..sample import Sample
 from ..utils import Code, anaCostModel
 from .tuner import Tuner, _run_jobs
 
+KEEP_BEST = 20          # best individuals seen in this call that rejoin the breeding pool after every generation
 
+
+# ---------------------------------------------------------------------------------------------- making children
+def _child_unconstrained(km, a, b, extra):
+    point, valid = km.crossover_and_mutate(a, b, extra)
+    return point, valid, {}
+
+
+def _child_constrained(km, a, b, keys):
+    point, valid = km.constrained_crossover_and_mutate(a, b, keys)
+    return point, valid, {}
+
+
+def _child_all_variables(km, a, b, feasible):
+    point, valid, violation = km.crossover_and_mutate_all(a, b, feasible)
+    return point, valid, {'violation': violation}
+
+
+def _child_sat_decoding(km, a, b, feasible):
+    point, valid = km.satdecoding_crossover_and_mutate(a, b, feasible)
+    return point, valid, {}
+
+
+def _child_sbx(km, a, b, feasible):
+    point, valid, violations = km.SBX_crossover_and_mutation(a, b, feasible)
+    return point, valid, {'violations': violations}
+
+
+BREED = {'Unconstrained': _child_unconstrained, 'Constrained': _child_constrained,
+         'UnconstrainedAll': _child_all_variables, 'SATDecoding': _child_sat_decoding, 'SBX': _child_sbx}
+
+
+def crossoverAndMutateSequential(kind, number, population, task, extra):
+    """``number`` children of random parent pairs (runs inside a forked worker when the tuner samples in parallel)."""
+    random.seed(int.from_bytes(os.urandom(8), "little"))
+    np.random.seed(int.from_bytes(os.urandom(4), "little"))
+    make = BREED[kind]
+    children = []
+    for _ in range(number if population else 0):
+        mother, father = random.choice(population), random.choice(population)
+        child = Sample(task)
+        point, valid, attrs = make(child.knob_manager, mother.knob_manager, father.knob_manager, extra)
+        for name, value in attrs.items():
+            setattr(child, name, value)
+        child.point, child.valid, child.stmt_code = point, bool(valid), Code(list(point))
+        children.append(child)
+    return children
+
+
+def crossoverAndMutateParallel(kind, number, population, task, parallel_num, extra, timeout=60):
+    share = -(-number // parallel_num)
+    return _run_jobs([Job(crossoverAndMutateSequential, (kind, share, population, task, extra), timeout)
+                      for _ in range(parallel_num)])
+
+
+def _offspring(config, kind, samples, task, extra):
+    if config.parallel:
+        return crossoverAndMutateParallel(kind, config.pop_num, samples, task, config.parallel_num, extra)
+    return crossoverAndMutateSequential(kind, config.pop_num, samples, task, extra)
+
+
+# ---------------------------------------------------------------------------------------------------- the tuners
 class GATuner(Tuner):
+    KIND = 'Unconstrained'
+
     def optimize(self, env, population, stat, s_time):
-        all_pop = [] + population
+        seen = list(population)
         for _ in range(self.config.iter_walks):
-            # nothing measured yet: the reference has no fitness to evolve on (ga_tuner.py:16-17); with an analytic
-            # estimate of the template the walks evolve on that, so the first measured batch is already a good one
-            if hasattr(self.cost_model, 'bst') and self.cost_model.bst is None and \
-                    not getattr(self.cost_model, 'has_prior', False):
+            if not self._has_fitness():
                 break
             self.inferKeyVariables(env, population)
-            population = self.RankPop(population)
-            population = self.Selection(population, self.config.select_num)
-            population = self.crossoverAndMutate(population, env.task)
-            all_pop += population
-            self.recordStat(all_pop, env, s_time, stat)
-            prevs = sorted(all_pop, key=lambda x: x.predict)[-20:]
-            population = population + prevs
-        self.removeInvalid(all_pop)
-        return population, all_pop
+            parents = self.Selection(self.RankPop(population), self.config.select_num)
+            population = self.crossoverAndMutate(parents, env.task)
+            seen += population
+            self.recordStat(seen, env, s_time, stat)
+            population = population + sorted(seen, key=lambda x: x.predict)[-KEEP_BEST:]
+        self.removeInvalid(seen)
+        return population, seen
 
+    def _has_fitness(self):
+        """Nothing measured yet: the reference has no fitness to evolve on and skips the walks (ga_tuner.py:16-17).
+        With an analytic estimate of the template the walks evolve on that, so the first measured batch is a good one."""
+        model = self.cost_model
+        untrained = hasattr(model, 'bst') and model.bst is None
+        return not untrained or getattr(model, 'has_prior', False)
+
+    # hooks of the generation step
     def inferKeyVariables(self, env, pop):
         return
 
@@ -45,85 +118,77 @@ class GATuner(Tuner):
     def Selection(self, pop, num):
         return self.RouletteWheelSelection(pop, num)
 
+    def breeding_extra(self, task):
+        return self.feasible
+
     def removeInvalid(self, all_pop):
         for sample in all_pop:
             if not sample.valid:
                 sample.predict = 0.0
 
+    def _score(self, children):
+        """Predicted score for the feasible children, zero for the others."""
+        good = [c for c in children if c.valid]
+        for child, p in zip(good, self.predict(good) if good else []):
+            child.predict = p
+        for child in children:
+            if not child.valid:
+                child.predict = 0
+        return children
+
     def crossoverAndMutate(self, samples, task):
-        if self.config.parallel:
-            res = crossoverAndMutateParallel('Unconstrained', self.config.pop_num, samples, task,
-                                             self.config.parallel_num, self.feasible)
-        else:
-            res = crossoverAndMutateSequential('Unconstrained', self.config.pop_num, samples, task, self.feasible)
-        vsamples = [s for s in res if s.valid]
-        if vsamples != []:
-            perfs = self.predict(vsamples)
-            for idx, sample in enumerate(vsamples):
-                sample.predict = perfs[idx]
-        for sample in res:
-            if not sample.valid:
-                sample.predict = 0
-        return res
+        return self._score(_offspring(self.config, self.KIND, samples, task, self.breeding_extra(task)))
 
 
-class CGATuner(GATuner):
+class _ConstrainedGA(GATuner):
+    """Children come out of the solver, so every one of them is feasible and no feasible-value table is needed."""
+    KIND = 'Constrained'
+
+    def check_feasible_exits(self, env, num=1e3):
+        return
+
+    def _random_keys(self, task):
+        names = list(task.knob_manager.solver.vals.keys())
+        random.shuffle(names)
+        return names[:int(self.config.crossover_key_ratio * len(names))]
+
+    def _score(self, children):
+        for child, p in zip(children, self.predict(children) if children else []):
+            child.predict = p
+        return children
+
+
+class CGATuner(_ConstrainedGA):
     def __init__(self, config):
         super().__init__(config)
+        self.key_variables = None
         # the last quarter of the measuring rounds refines the incumbents knob by knob: the fine knobs (issue order,
         # load spread, raster group, epilogue kind) move a good tile by a few percent, less than the cost model resolves
         self.refine_share = float(getattr(config, 'refine_share', 0.25))
 
-    def check_feasible_exits(self, env, num=1e3):
-        return
-
     def inferKeyVariables(self, env, pop):
-        vars_ = list(env.task.knob_manager.solver.vals.keys())
-        random.shuffle(vars_)
-        self.key_variables = vars_[:int(self.config.crossover_key_ratio * len(vars_))]
+        self.key_variables = self._random_keys(env.task)
 
-    def crossoverAndMutate(self, samples, task):
-        if hasattr(self, "key_variables") and self.key_variables is not None:
-            keys = self.key_variables
-        else:
-            keys = anaCostModel(self.cost_model, list(task.knob_manager.solver.vals.keys()))
-            keys = keys[:int(self.config.crossover_key_ratio * len(keys))]
-        if self.config.parallel:
-            res = crossoverAndMutateParallel('Constrained', self.config.pop_num, samples, task,
-                                             self.config.parallel_num, keys)
-        else:
-            res = crossoverAndMutateSequential('Constrained', self.config.pop_num, samples, task, keys)
-        perfs = self.predict(res)
-        for idx, sample in enumerate(res):
-            sample.predict = perfs[idx]
-        return res
+    def breeding_extra(self, task):
+        if self.key_variables is not None:
+            return self.key_variables
+        # no generation step has run yet: the variables the cost model weighs most (ga_tuner.py:79-83)
+        ranked = anaCostModel(self.cost_model, list(task.knob_manager.solver.vals.keys()))
+        return ranked[:int(self.config.crossover_key_ratio * len(ranked))]
 
 
-class RCGATuner(GATuner):
-    """CGA with fresh random key variables per call (ga_tuner.py:94-110)."""
+class RCGATuner(_ConstrainedGA):
+    """CGA with fresh random key variables per breeding call (ga_tuner.py:94-110)."""
 
-    def check_feasible_exits(self, env, num=1e3):
-        return
-
-    def crossoverAndMutate(self, samples, task):
-        keys = list(task.knob_manager.solver.vals.keys())
-        random.shuffle(keys)
-        keys = keys[:int(self.config.crossover_key_ratio * len(keys))]
-        if self.config.parallel:
-            res = crossoverAndMutateParallel('Constrained', self.config.pop_num, samples, task,
-                                             self.config.parallel_num, keys)
-        else:
-            res = crossoverAndMutateSequential('Constrained', self.config.pop_num, samples, task, keys)
-        perfs = self.predict(res)
-        for idx, sample in enumerate(res):
-            sample.predict = perfs[idx]
-        return res
+    def breeding_extra(self, task):
+        return self._random_keys(task)
 
 
 class SRGATuner(GATuner):
     """GA over all variables without constraint handling in the operators; constraint pressure comes from
     stochastic ranking: a bubble sort whose comparisons use the predicted score when both neighbours are feasible
-    or with probability ``pf``, and the total violation otherwise (ga_tuner.py:113-154)."""
+    or with probability ``PF``, and the total violation otherwise (ga_tuner.py:113-154)."""
+    KIND = 'UnconstrainedAll'
     SWEEPS, PF = 10, 0.45
 
     def Selection(self, pop, num):
@@ -136,72 +201,26 @@ class SRGATuner(GATuner):
             for j in range(len(order) - 1):
                 a, b = order[j], order[j + 1]
                 va, vb = a.violation or 0, b.violation or 0
-                if (va == 0 and vb == 0) or random.random() < self.PF:
-                    out_of_order = a.predict < b.predict
-                else:
-                    out_of_order = va > vb
-                if out_of_order:
+                by_score = (va == 0 and vb == 0) or random.random() < self.PF
+                if (a.predict < b.predict) if by_score else (va > vb):
                     order[j], order[j + 1] = b, a
                     swapped = True
             if not swapped:
                 break
         return order
 
-    def crossoverAndMutate(self, samples, task):
-        res = _offspring(self.config, 'UnconstrainedAll', samples, task, self.feasible)
-        perfs = self.predict(res)
-        for idx, sample in enumerate(res):
-            sample.predict = perfs[idx]
-        return res
+    def _score(self, children):
+        for child, p in zip(children, self.predict(children) if children else []):
+            child.predict = p
+        return children
 
 
 class SDGATuner(GATuner):
     """GA whose genotype is decoded into a feasible phenotype by repairing it with the solver
     (SAT-decoding, ga_tuner.py:157-166)."""
+    KIND = 'SATDecoding'
 
-    def crossoverAndMutate(self, samples, task):
-        res = _offspring(self.config, 'SATDecoding', samples, task, self.feasible)
-        perfs = self.predict(res)
-        for idx, sample in enumerate(res):
-            sample.predict = perfs[idx]
-        return res
-
-
-def _offspring(config, kind, samples, task, extra):
-    if config.parallel:
-        return crossoverAndMutateParallel(kind, config.pop_num, samples, task, config.parallel_num, extra)
-    return crossoverAndMutateSequential(kind, config.pop_num, samples, task, extra)
-
-
-def crossoverAndMutateParallel(kind, number, population, task, parallel_num, extra, timeout=60):
-    work_load = int((number + parallel_num - 1) // parallel_num)
-    jobs = [Job(crossoverAndMutateSequential, (kind, work_load, population, task, extra), timeout)
-            for _ in range(parallel_num)]
-    return _run_jobs(jobs)
-
-
-def crossoverAndMutateSequential(kind, number, population, task, extra):
-    random.seed(int.from_bytes(os.urandom(8), "little"))
-    np.random.seed(int.from_bytes(os.urandom(4), "little"))
-    ret = []
-    if len(population) == 0:
-        return ret
-    for _ in range(number):
-        m1 = population[random.randint(0, len(population) - 1)]
-        m2 = population[random.randint(0, len(population) - 1)]
-        child = Sample(task)
-        if kind == 'Constrained':
-            point, valid = child.knob_manager.constrained_crossover_and_mutate(m1.knob_manager, m2.knob_manager, extra)
-        elif kind == 'UnconstrainedAll':
-            point, valid, child.violation = child.knob_manager.crossover_and_mutate_all(m1.knob_manager, m2.knob_manager, extra)
-        elif kind == 'SATDecoding':
-            point, valid = child.knob_manager.satdecoding_crossover_and_mutate(m1.knob_manager, m2.knob_manager, extra)
-        elif kind == 'SBX':
-            point, valid, child.violations = child.knob_manager.SBX_crossover_and_mutation(m1.knob_manager, m2.knob_manager, extra)
-        else:
-            point, valid = child.knob_manager.crossover_and_mutate(m1.knob_manager, m2.knob_manager, extra)
-        child.point = point
-        child.valid = bool(valid)
-        child.stmt_code = Code(list(point))
-        ret.append(child)
-    return ret
+    def _score(self, children):
+        for child, p in zip(children, self.predict(children) if children else []):
+            child.predict = p
+        return children

@@ -266,7 +266,7 @@ def test_baseline_tuners_run_and_only_measure_feasible_points(tmp_path, method):
     np.random.seed(1)
     env.tune("T1")
     rows = [json.loads(l) for l in open(os.path.join(env.config.log_dir, "records.txt"))]
-    assert 8 <= len(rows) <= 40           # two full rounds of 16 plus the 24 % 16 remainder round (tuner.py:50-58)
+    assert 8 <= len(rows) <= 40           # one full round of 16 plus the 24 % 16 remainder round
     solver = env.task.knob_manager.solver
     for r in rows:
         assert solver.SATScore(r["param"]) == 0
