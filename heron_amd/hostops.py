@@ -74,69 +74,96 @@ def _pad_last(t, to):
     return torch.nn.functional.pad(t, (0, to - t.shape[-1])).contiguous()      # one pass
 
 
-def _prep_identity(info, A, Bm):
-    return A, Bm
+# Every adapter has two halves: ``act`` maps the activation input(s) to the kernel's A operand and is needed on every
+# call; ``const`` maps the constant input (filter, vector) - or nothing but the shapes - to the kernel's B operand and is
+# needed once per set of weights (run_operator caches it when asked to).
+def _act_identity(info, A, Bm):
+    return A
 
 
-def _prep_gemv(info, A, b):
-    K = info['gemm_view']['K']
-    Bp = torch.zeros((info['gemm_view']['N'], K), dtype=b.dtype, device=b.device)
+def _const_identity(info, A, Bm):
+    return Bm
+
+
+def _act_pad_k(info, A, *_):
+    return _pad_last(A, info['gemm_view']['K'])
+
+
+def _const_gemv(info, A, b):
+    g = info['gemm_view']
+    Bp = torch.zeros((g['N'], g['K']), dtype=b.dtype, device=b.device)
     Bp[0, :b.shape[-1]] = b.reshape(-1)
-    return _pad_last(A, K), Bp
+    return Bp
 
 
-def _prep_scan(info, A):
+def _const_scan(info, A):
     g = info['gemm_view']
     n = torch.arange(g['N'], device=A.device).unsqueeze(1)
     k = torch.arange(g['K'], device=A.device).unsqueeze(0)
     T = (n > k).to(torch.float16 if info['kind'] == 'f16' else torch.int8)
     T[:, A.shape[-1]:] = 0
-    return _pad_last(A, g['K']), T
+    return T
 
 
-def _prep_mean(info, In):
+def _act_mean(info, In, *_):
+    N, C, H, W = In.shape
+    return _pad_last(In.permute(1, 0, 2, 3).reshape(C, N * H * W), info['gemm_view']['K'])
+
+
+def _const_mean(info, In, *_):
     g = info['gemm_view']
     N, C, H, W = In.shape
-    A = In.permute(1, 0, 2, 3).reshape(C, N * H * W)
     Bm = torch.zeros((g['N'], g['K']), dtype=In.dtype, device=In.device)
     Bm[0, :N * H * W] = 1.0 / (N * H * W)
-    return _pad_last(A, g['K']), Bm
+    return Bm
 
 
-def _prep_var(info, In, Mean):
+def _act_var(info, In, Mean):
     d = In - Mean
-    return _prep_mean(info, d * d)
+    return _act_mean(info, d * d)
 
 
 def _cpad(info):
     return info['conv']['CI']
 
 
-def _prep_c1d_nwc(info, X, F):            # (N,W,CI), (K,CI,CO)
-    Xk = _pad_last(X, _cpad(info)).unsqueeze(1)
-    Wk = _pad_last(F.permute(2, 0, 1), _cpad(info)).unsqueeze(1)
-    return Xk, Wk.contiguous()
+def _act_c1d_nwc(info, X, F):             # (N,W,CI)
+    return _pad_last(X, _cpad(info)).unsqueeze(1)
 
 
-def _prep_c1d_ncw(info, X, F):            # (N,CI,W), (CO,CI,KW)
-    Xk = _pad_last(X.permute(0, 2, 1), _cpad(info)).unsqueeze(1)
-    Wk = _pad_last(F.permute(0, 2, 1), _cpad(info)).unsqueeze(1)
-    return Xk, Wk.contiguous()
+def _const_c1d_nwc(info, X, F):           # (K,CI,CO)
+    return _pad_last(F.permute(2, 0, 1), _cpad(info)).unsqueeze(1).contiguous()
 
 
-def _prep_c2d_nchw(info, X, F):           # (N,CI,H,W), (CO,CI,KH,KW)
-    return _pad_last(X.permute(0, 2, 3, 1), _cpad(info)), _pad_last(F.permute(0, 2, 3, 1), _cpad(info))
+def _act_c1d_ncw(info, X, F):             # (N,CI,W)
+    return _pad_last(X.permute(0, 2, 1), _cpad(info)).unsqueeze(1)
 
 
-def _prep_c2d_krsc(info, X, F):           # (N,H,W,CI), (CO,KH,KW,CI) with CI short of a whole 16-byte chunk
-    return _pad_last(X, _cpad(info)), _pad_last(F, _cpad(info))
+def _const_c1d_ncw(info, X, F):           # (CO,CI,KW)
+    return _pad_last(F.permute(0, 2, 1), _cpad(info)).unsqueeze(1).contiguous()
 
 
-def _prep_c2d_hwio(info, X, F):           # (N,H,W,CI), (KH,KW,CI,CO)
-    return _pad_last(X, _cpad(info)), _pad_last(F.permute(3, 0, 1, 2), _cpad(info))
+def _act_nchw(info, X, F):                # (N,CI,H,W)
+    return _pad_last(X.permute(0, 2, 3, 1), _cpad(info))
 
 
-def _prep_c3d_ndhwc(info, X, F):          # (N,D,H,W,CI), (KD,KH,KW,CI,CO)
+def _const_oihw(info, X, F):              # (CO,CI,KH,KW)
+    return _pad_last(F.permute(0, 2, 3, 1), _cpad(info))
+
+
+def _act_nhwc(info, X, F):                # (N,H,W,CI), CI possibly short of a whole 16-byte chunk
+    return _pad_last(X, _cpad(info))
+
+
+def _const_krsc(info, X, F):              # (CO,KH,KW,CI)
+    return _pad_last(F, _cpad(info))
+
+
+def _const_hwio(info, X, F):              # (KH,KW,CI,CO)
+    return _pad_last(F.permute(3, 0, 1, 2), _cpad(info))
+
+
+def _act_c3d_ndhwc(info, X, F):           # (N,D,H,W,CI)
     dp = info['depth']
     N, D, H, W, CI = X.shape
     KD, DO, sd, pd, dd = dp['KD'], dp['DO'], dp['stride'], dp['pad'], dp['dil']
@@ -145,16 +172,25 @@ def _prep_c3d_ndhwc(info, X, F):          # (N,D,H,W,CI), (KD,KH,KW,CI,CO)
     Xp[:, pd:pd + D, :, :, :CI] = X
     # depth taps side by side on the channel axis: channel block kd of output slice z is input slice z*sd + kd*dd
     cols = torch.stack([Xp[:, kd * dd: kd * dd + (DO - 1) * sd + 1: sd] for kd in range(KD)], dim=4)
-    Xk = cols.reshape(N * DO, H, W, KD * cip).contiguous()
+    return cols.reshape(N * DO, H, W, KD * cip).contiguous()
+
+
+def _const_c3d_dhwio(info, X, F):         # (KD,KH,KW,CI,CO)
+    KD = info['depth']['KD']
+    cip = info['conv']['CI'] // KD
     Fp = _pad_last(F.permute(4, 1, 2, 0, 3), cip)                    # (CO,KH,KW,KD,cip)
-    return Xk, Fp.reshape(Fp.shape[0], Fp.shape[1], Fp.shape[2], KD * cip).contiguous()
+    return Fp.reshape(Fp.shape[0], Fp.shape[1], Fp.shape[2], KD * cip).contiguous()
 
 
-def _prep_c3d_ncdhw(info, X, F):          # (N,CI,D,H,W), (CO,CI,KD,KH,KW)
-    return _prep_c3d_ndhwc(info, X.permute(0, 2, 3, 4, 1), F.permute(2, 3, 4, 1, 0))
+def _act_c3d_ncdhw(info, X, F):           # (N,CI,D,H,W)
+    return _act_c3d_ndhwc(info, X.permute(0, 2, 3, 4, 1), F)
 
 
-def _prep_t2d_nchw(info, X, F):           # (N,CI,H,W), (CO,CI,KH,KW)
+def _const_c3d_oidhw(info, X, F):         # (CO,CI,KD,KH,KW)
+    return _const_c3d_dhwio(info, X, F.permute(2, 3, 4, 1, 0))
+
+
+def _act_t2d_nchw(info, X, F):            # (N,CI,H,W): zero-expanded by the stride and padded, channels last
     t = info['transposed']
     c = info['conv']
     N, CI, H, W = X.shape
@@ -163,22 +199,28 @@ def _prep_t2d_nchw(info, X, F):           # (N,CI,H,W), (CO,CI,KH,KW)
     left = (c['KW'] - 1) * t['dil'] - t['pad']
     Xe = torch.zeros((N, c['H'], c['W'], c['CI']), dtype=X.dtype, device=X.device)
     Xe[:, top: top + (H - 1) * s + 1: s, left: left + (W - 1) * s + 1: s, :CI] = X.permute(0, 2, 3, 1)
-    return Xe, _pad_last(F.permute(0, 2, 3, 1), c['CI'])
+    return Xe
 
 
-def _prep_dep(info, X, F):                # (N,C,H,W), (K,3,3): the 3x3 windows as 4x4 = 16 taps per pixel and channel
+def _act_dep(info, X, F):                 # (N,C,H,W): the 3x3 windows as 4x4 = 16 taps per pixel and channel
     d = info['dep']
     N, C, H, W = X.shape
-    s, p, HO, WO, mult, NP = d['stride'], d['pad'], d['HO'], d['WO'], d['mult'], d['NP']
+    s, p, HO, WO = d['stride'], d['pad'], d['HO'], d['WO']
     Xp = torch.zeros((N, C, H + 2 * p + 1, W + 2 * p + 1), dtype=X.dtype, device=X.device)
     Xp[:, :, p:p + H, p:p + W] = X
     A = torch.zeros((C, N, HO, WO, 4, 4), dtype=X.dtype, device=X.device)
     for r in range(3):
         for q in range(3):
             A[:, :, :, :, r, q] = Xp[:, :, r: r + (HO - 1) * s + 1: s, q: q + (WO - 1) * s + 1: s].permute(1, 0, 2, 3)
+    return A.reshape(C, N * HO * WO, 16)
+
+
+def _const_dep(info, X, F):               # (K,3,3)
+    d = info['dep']
+    C, mult, NP = X.shape[1], d['mult'], d['NP']
     Bm = torch.zeros((C, NP, 4, 4), dtype=F.dtype, device=F.device)
     Bm[:, :mult, :3, :3] = F.reshape(C, mult, 3, 3)
-    return A.reshape(C, N * HO * WO, 16), Bm.reshape(C, NP, 16)
+    return Bm.reshape(C, NP, 16)
 
 
 def _fin_dep(info, Cm):                   # (C, N*HO*WO, NP) -> (N, C, NP, HO, WO)
@@ -212,20 +254,21 @@ def _fin_c3d_ncdhw(info, C):              # -> (N,CO,DO,HO,WO)
 
 
 ADAPTERS = {
-    'identity': (_prep_identity, _fin_identity),
-    'gemv': (_prep_gemv, _fin_identity),
-    'scan': (_prep_scan, _fin_identity),
-    'mean': (_prep_mean, _fin_identity),
-    'var': (_prep_var, _fin_identity),
-    'c1d_nwc': (_prep_c1d_nwc, _fin_c1d_nwc),
-    'c1d_ncw': (_prep_c1d_ncw, _fin_c1d_ncw),
-    'c2d_nchw': (_prep_c2d_nchw, _fin_nchw),
-    'c2d_hwio': (_prep_c2d_hwio, _fin_identity),
-    'c2d_krsc': (_prep_c2d_krsc, _fin_identity),
-    'c3d_ndhwc': (_prep_c3d_ndhwc, _fin_c3d_ndhwc),
-    'c3d_ncdhw': (_prep_c3d_ncdhw, _fin_c3d_ncdhw),
-    't2d_nchw': (_prep_t2d_nchw, _fin_nchw),
-    'dep': (_prep_dep, _fin_dep),
+    # name: (activation half, constant half, result reorder)
+    'identity': (_act_identity, _const_identity, _fin_identity),
+    'gemv': (_act_pad_k, _const_gemv, _fin_identity),
+    'scan': (_act_pad_k, _const_scan, _fin_identity),
+    'mean': (_act_mean, _const_mean, _fin_identity),
+    'var': (_act_var, _const_mean, _fin_identity),
+    'c1d_nwc': (_act_c1d_nwc, _const_c1d_nwc, _fin_c1d_nwc),
+    'c1d_ncw': (_act_c1d_ncw, _const_c1d_ncw, _fin_c1d_ncw),
+    'c2d_nchw': (_act_nchw, _const_oihw, _fin_nchw),
+    'c2d_hwio': (_act_nhwc, _const_hwio, _fin_identity),
+    'c2d_krsc': (_act_nhwc, _const_krsc, _fin_identity),
+    'c3d_ndhwc': (_act_c3d_ndhwc, _const_c3d_dhwio, _fin_c3d_ndhwc),
+    'c3d_ncdhw': (_act_c3d_ncdhw, _const_c3d_oidhw, _fin_c3d_ncdhw),
+    't2d_nchw': (_act_t2d_nchw, _const_oihw, _fin_nchw),
+    'dep': (_act_dep, _const_dep, _fin_dep),
 }
 
 
@@ -234,13 +277,21 @@ ADAPTERS = {
 ACTIVATION_AS_IS = ('identity', 'c1d_nwc', 'c2d_hwio', 'c2d_krsc')
 
 
-def run_operator(mod, info, inputs, group_m=8, split_k=0):
+def prepare_constant(info, inputs):
+    """The kernel's B operand of an operator: the reordered / padded filter or the generated right-hand side.  It
+    depends on the weights and the shapes only, so a caller with fixed weights prepares it once."""
+    return ADAPTERS[info.get('adapter', 'identity')][1](info, *inputs)
+
+
+def run_operator(mod, info, inputs, group_m=8, split_k=0, constant=None):
     """Runs one operator of the registry on device tensors given in the reference's own layouts.
 
     ``info`` is the dictionary the operator definition handed to ``ctx.set_info``; ``mod`` an instance of the
-    template that matches its kind and operator."""
-    prep, fin = ADAPTERS[info.get('adapter', 'identity')]
-    A, Bm = prep(info, *inputs)
+    template that matches its kind and operator; ``constant`` a B operand from ``prepare_constant`` (made here when
+    absent)."""
+    act, const, fin = ADAPTERS[info.get('adapter', 'identity')]
+    A = act(info, *inputs)
+    Bm = const(info, *inputs) if constant is None else constant
     if info['operator'] == 'conv2d_nhwc':
         c = info['conv']
         C = conv2d_nhwc(mod, A, Bm, (c['stride'], c['stride_w']), (c['pad'], c['pad_w']), (c['dil'], c['dil_w']),

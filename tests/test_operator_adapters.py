@@ -27,8 +27,10 @@ def through_adapter(name, args, inputs):
     c = Ctx()
     out = getOpFromName(name)(c, *args, "float16", "float16")
     info = c.info
-    prep, fin = hostops.ADAPTERS[info['adapter']]
-    A, Bm = prep(info, *[torch.from_numpy(np.ascontiguousarray(x)) for x in inputs])
+    act, const, fin = hostops.ADAPTERS[info['adapter']]
+    tensors = [torch.from_numpy(np.ascontiguousarray(x)) for x in inputs]
+    A, Bm = act(info, *tensors), const(info, *tensors)
+    assert torch.equal(Bm, hostops.prepare_constant(info, tensors))
     g = info['gemm_view']
     if info['operator'] == 'conv2d_nhwc':
         cv = info['conv']
@@ -98,8 +100,8 @@ def test_depthwise(s, p, mult):
     X, F = rnd((2, 6, 9, 8), 16), rnd((6 * mult, 3, 3), 17)
     c = Ctx()
     out = getOpFromName("dep")(c, 2, 9, 8, 6, 6 * mult, 3, 3, s, p, 1, "float16", "float16")
-    prep, fin = hostops.ADAPTERS[c.info['adapter']]
-    A, Bm = prep(c.info, torch.from_numpy(X), torch.from_numpy(F))
+    act, const, fin = hostops.ADAPTERS[c.info['adapter']]
+    A, Bm = act(c.info, torch.from_numpy(X), torch.from_numpy(F)), const(c.info, torch.from_numpy(X), torch.from_numpy(F))
     g = c.info['gemm_view']
     assert tuple(A.shape) == (g['batch'], g['M'], g['K']) and tuple(Bm.shape) == (g['batch'], g['N'], g['K'])
     C = oracle.bmm_f32(A.numpy(), Bm.numpy())
