@@ -143,6 +143,7 @@ SYMBOLS = {
     "hrn_probe_mfma": (_i, [_i, _i, _i, ctypes.POINTER(_d), _vp]),
     "hrn_probe_copy": (_i, [_vp, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_probe_launch": (_i, [_i, _i, ctypes.POINTER(_d), _vp]),
+    "hrn_pad_rows": (_i, [_vp, _vp, ctypes.c_size_t, _i, _i, _i, _vp]),
     "hrn_probe_read": (_i, [_vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_last_error": (ctypes.c_char_p, []),
     "hrn_version": (ctypes.c_char_p, []),
@@ -238,6 +239,11 @@ def probe_launch(grid=256, repeat=2000, stream=0):
     out = ctypes.c_double()
     _check(lib().hrn_probe_launch(grid, repeat, ctypes.byref(out), stream))
     return out.value
+
+
+def pad_rows(src_ptr, dst_ptr, rows, c, cp, elem_bytes, stream=0):
+    """Zero-pads rows of c elements to cp elements (device pointers, dst holds rows * cp elements)."""
+    _check(lib().hrn_pad_rows(src_ptr, dst_ptr, rows, c, cp, elem_bytes, stream))
 
 
 def probe_read(src_ptr, nbytes, repeat=10, stream=0):

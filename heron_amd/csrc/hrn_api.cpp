@@ -622,6 +622,28 @@ __global__ void __launch_bounds__(256) probe_copy_kernel(const pv4i* __restrict_
     for (; i < n16; i += stride) dst[i] = src[i];
 }
 
+// One lane per row: copies `c` elements of ES bytes and zero-fills up to `cp` elements, writing whole 16-byte words.
+template <int ES>
+__global__ void __launch_bounds__(256) pad_rows_kernel(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst,
+                                                       size_t rows, int c, int cp) {
+    const size_t row = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= rows) return;
+    const unsigned char* in = src + row * (size_t)c * ES;
+    pv4i* out = (pv4i*)(dst + row * (size_t)cp * ES);
+    const int words = cp * ES / 16, live = c * ES;
+    for (int w = 0; w < words; ++w) {
+        unsigned int q[4] = {0u, 0u, 0u, 0u};
+        for (int b = 0; b < 16; b += ES) {
+            const int at = w * 16 + b;
+            if (at < live) {
+                const unsigned int v = ES == 2 ? (unsigned int)*(const unsigned short*)(in + at) : (unsigned int)in[at];
+                q[b / 4] |= v << (8 * (b % 4));
+            }
+        }
+        out[w] = pv4i{(int)q[0], (int)q[1], (int)q[2], (int)q[3]};
+    }
+}
+
 // streams `n16` 16-byte words through every lane without storing anything: the read-only counterpart of the copy probe
 __global__ void __launch_bounds__(256) probe_read_kernel(const pv4i* __restrict__ src, size_t n16) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -644,6 +666,19 @@ __global__ void __launch_bounds__(256) probe_empty_kernel(int* sink) {
 }  // namespace
 
 extern "C" {
+
+int hrn_pad_rows(const void* src, void* dst, size_t rows, int c, int cp, int elem_bytes, void* stream) {
+    if (!src || !dst || c < 1 || cp < c || (elem_bytes != 1 && elem_bytes != 2) || (cp * elem_bytes) % 16 || rows > ((size_t)1 << 40))
+        return fail(HRN_E_BADPARAM, "pad_rows: %d -> %d elements of %d bytes (the padded row must be whole 16-byte words)", c, cp, elem_bytes);
+    if (rows == 0) return HRN_OK;
+    const unsigned grid = (unsigned)((rows + 255) / 256);
+    hipStream_t st = (hipStream_t)stream;
+    if (elem_bytes == 2) pad_rows_kernel<2><<<grid, 256, 0, st>>>((const unsigned char*)src, (unsigned char*)dst, rows, c, cp);
+    else pad_rows_kernel<1><<<grid, 256, 0, st>>>((const unsigned char*)src, (unsigned char*)dst, rows, c, cp);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HRN_E_LAUNCH, "pad_rows: %s", hipGetErrorString(e));
+    return HRN_OK;
+}
 
 int hrn_probe_read(const void* src, size_t bytes, int repeat, double* gbs_out, void* stream) {
     if (!src || !gbs_out || bytes < 16 || bytes % 16 || repeat < 1) return fail(HRN_E_BADPARAM, "probe arguments");

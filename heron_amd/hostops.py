@@ -69,9 +69,15 @@ def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8, split_k
 # tensors, in the reference's layouts, to the template's operands (A (M,K) / B (N,K), or NHWC / KRSC) and
 # maps the result back.  They only move, pad or generate data; every multiply-accumulate is the kernel's.
 def _pad_last(t, to):
-    if t.shape[-1] == to:
+    """``t`` with its last axis zero-padded to ``to`` elements, contiguous."""
+    c = t.shape[-1]
+    if c == to:
         return t.contiguous()
-    return torch.nn.functional.pad(t, (0, to - t.shape[-1])).contiguous()      # one pass
+    if t.is_cuda and t.is_contiguous() and t.element_size() in (1, 2) and (to * t.element_size()) % 16 == 0:
+        out = torch.empty(t.shape[:-1] + (to,), dtype=t.dtype, device=t.device)
+        B.pad_rows(t.data_ptr(), out.data_ptr(), t.numel() // c, c, to, t.element_size(), _stream())
+        return out
+    return torch.nn.functional.pad(t, (0, to - c)).contiguous()
 
 
 # Every adapter has two halves: ``act`` maps the activation input(s) to the kernel's A operand and is needed on every

@@ -162,9 +162,11 @@ class CGATuner(_ConstrainedGA):
     def __init__(self, config):
         super().__init__(config)
         self.key_variables = None
+
+    def refinement_share(self):
         # the last quarter of the measuring rounds refines the incumbents knob by knob: the fine knobs (issue order,
         # load spread, raster group, epilogue kind) move a good tile by a few percent, less than the cost model resolves
-        self.refine_share = float(getattr(config, 'refine_share', 0.25))
+        return float(getattr(self.config, 'refine_share', 0.25))
 
     def inferKeyVariables(self, env, pop):
         self.key_variables = self._random_keys(env.task)

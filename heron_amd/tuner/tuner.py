@@ -36,9 +36,11 @@ class Tuner:
         self.total_sample_time = 0
         self.total_measure_time = 0
         self.feasible = None
-        # share of the measuring rounds, at the end of a run, whose candidates are the one-knob neighbours of the best
-        # measured points (constrained tuners switch it on); the reference has no such phase
-        self.refine_share = 0.0
+
+    def refinement_share(self):
+        """Share of the measuring rounds, at the end of a run, whose candidates are the one-knob neighbours of the best
+        measured points (the constrained GA switches it on); the reference has no such phase."""
+        return 0.0
 
     # ------------------------------------------------------------------------------------------------ cost model
     def buildCostModel(self, task):
@@ -104,7 +106,7 @@ class Tuner:
         # adds a round of its own in front of the remainder, a run measures max_trials points, not up to a round more
         quotas = [per_round] * full + [rest]
         measuring = full + (1 if rest else 0)
-        refine_from = measuring - (int(self.refine_share * measuring + 0.5) if measuring >= 3 else 0)
+        refine_from = measuring - (int(self.refinement_share() * measuring + 0.5) if measuring >= 3 else 0)
         population, stat = [], []
         print("= ---- Tuning : Trials %d, Rounds %d ---- =" % (self.config.max_trials, len(quotas)))
         for iter_no, quota in enumerate(quotas):

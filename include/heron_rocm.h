@@ -218,6 +218,14 @@ int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, co
                   void* flush_buf, size_t flush_bytes, int repeat, double* costs_out, void* stream);
 
 /*
+ * Channel padding pre-stage: copies `rows` rows of `c` elements (1 or 2 bytes each) from `src` to rows of `cp`
+ * elements in `dst`, zero-filling the tail; cp * elem_bytes must be a multiple of 16.  Replaces the `pad` /
+ * layout stages the reference inlines in front of its tensorized conv (ops/cuda/conv2d.py:160-170) for inputs whose
+ * channel count is short of a 16-byte chunk (the 3-channel stem).  Both buffers are caller-owned device memory.
+ */
+int hrn_pad_rows(const void* src, void* dst, size_t rows, int c, int cp, int elem_bytes, void* stream);
+
+/*
  * Roofline probes (no counterpart in the reference, which never relates a timing to a hardware
  * limit).  hrn_probe_mfma times a register-resident loop of independent MFMAs of the given
  * dtype/shape on every CU and returns dense T(FL)OP/s (random_operands != 0 feeds operands with the

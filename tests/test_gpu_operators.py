@@ -127,6 +127,9 @@ def test_conv2d_nchw_dilated_and_transposed(dtype, hrn):
         info, _ = declare("c2d", [N, H, W, CI, CO, KH, KW, s, p, d], dtype)
         ref = oracle.conv2d_nhwc_f32(X, F, s, p, d) if f16 else oracle.conv2d_nhwc_u8s8s32(X, F, s, p, d)
         check(hostops.run_operator(module(info), info, [dev(X), dev(F)]), ref, f16)
+        # the same call with the filter prepared once, as the measurer and a caller with fixed weights do
+        weights = hostops.prepare_constant(info, [dev(X), dev(F)])
+        check(hostops.run_operator(module(info), info, [dev(X), dev(F)], constant=weights), ref, f16)
     for (N, H, W, CI, CO, KH, KW, s, p, d) in [(2, 20, 20, 16, 16, 3, 3, 1, 2, 2), (1, 17, 13, 8, 12, 3, 3, 2, 3, 3)]:
         X, F = rnd((N, H, W, CI), 9, a_dt), rnd((KH, KW, CI, CO), 10, b_dt)
         print("dil", dtype, (N, H, W, CI, CO, KH, KW, s, p, d), flush=True)
@@ -181,3 +184,22 @@ def test_depthwise_conv(dtype, hrn):
         print("dep", dtype, (N, H, W, C, K, s, p), flush=True)
         info, _ = declare("dep", [N, H, W, C, K, 3, 3, s, p, 1], dtype)
         check(hostops.run_operator(module(info), info, [dev(X), dev(F)]), oracle.depthwise_conv2d_ref(X, F, s, p), f16)
+
+
+def test_pad_rows_kernel(hrn):
+    """The channel-padding pre-stage of the library against torch's pad, both element sizes, odd row counts."""
+    import torch
+    for dtype, c, cp in [(torch.float16, 3, 8), (torch.float16, 20, 24), (torch.uint8, 3, 16), (torch.int8, 17, 32), (torch.float16, 1, 8)]:
+        for rows in (1, 255, 4097):
+            if dtype == torch.float16:
+                t = torch.randn((rows, c), device="cuda").to(dtype)
+            else:
+                t = torch.randint(0, 100, (rows, c), device="cuda").to(dtype)
+            out = torch.full((rows, cp), 7, dtype=dtype, device="cuda")
+            B.pad_rows(t.data_ptr(), out.data_ptr(), rows, c, cp, t.element_size(), torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
+            assert torch.equal(out, torch.nn.functional.pad(t, (0, cp - c))), (dtype, c, cp, rows)
+    x = torch.randn((2, 5, 7, 3), device="cuda").half()
+    assert torch.equal(hostops._pad_last(x, 8), torch.nn.functional.pad(x, (0, 5)))
+    with pytest.raises(B.HeronRocmError):
+        B.pad_rows(x.data_ptr(), x.data_ptr(), 4, 3, 6, 2, 0)            # 12-byte rows are not whole 16-byte words

@@ -410,3 +410,33 @@ def test_shipped_tuned_records_reinstantiate(rel, op, shape, dtype):
     best = max(rows, key=lambda r: r["perf"])
     stage = s.info['stage_name']
     assert s.params['bm'] == best["param"]["V#ST:%s,AX:None,VA:block_m" % stage]
+
+
+def test_refinement_rounds_measure_one_knob_neighbours(tmp_path, capsys):
+    """CGA spends the last quarter of its measuring rounds on the one-knob neighbourhood of the best measured points:
+    every neighbour is a feasible point that differs from one of the incumbents in exactly one knob."""
+    env = make_env(tmp_path, method="CGA", trials=64)
+    np.random.seed(2)
+    random.seed(2)
+    env.tune("T1")
+    out = capsys.readouterr().out
+    assert out.count("refinement round:") == 1                       # 4 measuring rounds of 16 -> the last one
+    tuner = env.tuner if hasattr(env, "tuner") else None
+    from heron_amd.tuner.ga_tuner import CGATuner
+    t = tuner or CGATuner(env.config)
+    t.buildCostModel(env.task)
+    near = t.incumbent_neighbours(env, top=2)
+    assert len(near) >= 10
+    solver = env.task.knob_manager.solver
+    names = env.task.knob_manager.knob_names
+    tops = [s.knob_manager.solved_knob_vals_genotype for s in t.history_topk_samples(env, 2)]
+    for s in near:
+        vals = s.knob_manager.solved_knob_vals_phenotype
+        assert s.valid and solver.SATScore(vals) == 0
+        assert min(sum(1 for n in names if vals[n] != top[n]) for top in tops) == 1
+    # the share is a config key; 0 gives the plain loop
+    env0 = make_env(tmp_path / "plain", method="CGA", trials=48)
+    env0.config.refine_share = 0
+    (tmp_path / "plain").mkdir(exist_ok=True)
+    env0.tune("T1")
+    assert "refinement round:" not in capsys.readouterr().out
