@@ -258,8 +258,8 @@ class KnobManager:
                 known[key] = [m1.solved_knob_vals_genotype[key], m2.solved_knob_vals_genotype[key]]
         try:
             valid, res = self.randSample(known)
-        except AssertionError:
-            # the two parents cannot be combined on these keys: fall back to a fresh sample
+        except (AssertionError, RuntimeError):
+            # the two parents cannot be combined on these keys (or the search gave up): fall back to a fresh sample
             valid, res = self.randSample({})
         return res, valid
 
@@ -340,7 +340,10 @@ class KnobManager:
         preserve_num = int(ratio * len(keys))
         positions = set(np.random.choice(len(keys), preserve_num, replace=False).tolist())
         known = {key: [knob_manager.solved_knob_vals_genotype[key]] for idx, key in enumerate(keys) if idx in positions}
-        valid, res = self.randSample(known)
+        try:
+            valid, res = self.randSample(known)
+        except RuntimeError:
+            valid, res = self.randSample({})        # the search gave up on this subset: a fresh point instead
         return res, valid
 
     def random_walk(self, knob_manager, feasible):

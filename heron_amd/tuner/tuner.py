@@ -296,7 +296,10 @@ def constrained_random_sample_sequential(task, number, config):
     out = []
     for _ in range(number):
         sample = Sample(task)
-        valid, point = sample.knob_manager.randSample({})
+        try:
+            valid, point = sample.knob_manager.randSample({})
+        except RuntimeError:
+            continue                # the search gave up on this draw; the rest of the batch is still worth having
         out.append(_finish(sample, point, valid))
     return out
 
