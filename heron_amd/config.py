@@ -24,7 +24,7 @@ DEFAULTS = {
     # unconstrained tuners: per-variable feasible value sets from this many random feasible points (tuner.py:115-144)
     'feasible_file_path': 'feasible.json', 'feasible_samples': 1000,
     # cross-task cost model: rounds of run_with_pretrained (the reference reads it, tuner.py:36, but never defines it)
-    'search_generations': 4, 'pretrained_records': (),
+    'search_generations': 4, 'pretrained_records': (), 'pretrained_model': '',
     # what a JSON file normally supplies
     'opt_method': 'CGA', 'max_trials': 32, 'runner_number': 3, 'runner_repeat': 4, 'runner_timeout': 50,
     'build_timeout': 50, 'in_dtype': 'float16', 'out_dtype': 'float16', 'cases': (),

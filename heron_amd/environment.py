@@ -83,7 +83,16 @@ class Env:
         self.runner.measure_batch = create_measure_batch(self.task, self.runner.measure_option)
         with open(os.path.join(self.config.log_dir, 'schedule.py'), 'w') as out:
             out.write(self.task.sched_desc)
-        if pretrained or self.config.pretrained_records:
+        if getattr(self.config, 'pretrained_model', ''):
+            # an attention cost model fitted beforehand on the records of other tasks (tests/pretrain/train_model.py),
+            # used as it is: the flow of pretrain/tune_with_pretrained.py:30-35 of the reference
+            from .pretrain import AttentionCostModel
+            model = AttentionCostModel().load(self.config.pretrained_model)
+            print("pre-trained attention cost model: %s (%d variable names)" % (self.config.pretrained_model,
+                                                                               model.vocab.size("name") - 1))
+            self.tuner.setPretrainedModel(model)
+            result = self.tuner.run_with_pretrained(self)
+        elif pretrained or self.config.pretrained_records:
             from .model import PretrainedCostModel
             model = PretrainedCostModel(self.task, self.config)
             n = model.fit_from_records(self.config.pretrained_records, len(self.task.knob_manager.solver.vals))

@@ -106,6 +106,9 @@ if __name__ == '__main__':
     parser.add_argument("--cold", action="store_true",
                         help="time every launch from flushed caches (the runner's enable_cpu_cache_flush of "
                              "tests/quick_start/dlboost/run.py:89-96, on the GPU): for cases bound by HBM traffic")
+    parser.add_argument("--pretrained-model", type=str, default="",
+                        help="attention cost model saved by tests/pretrain/train_model.py: the search is steered by it "
+                             "from the first round and it is not re-trained (pretrain/tune_with_pretrained.py)")
     parser.add_argument("--pretrained", type=str, default="",
                         help="comma separated records.txt files of earlier tasks of the same operator: steer the search "
                              "with a cost model fitted on them instead of training one from scratch")
@@ -118,6 +121,7 @@ if __name__ == '__main__':
     config.tuned = args.tuned
     config.verbose = args.verbose
     config.pretrained_records = [p for p in args.pretrained.split(",") if p]
+    config.pretrained_model = os.path.abspath(args.pretrained_model) if args.pretrained_model else ""
     config.cold = args.cold
     runner = HeronRunner.LocalRunner(number=config.runner_number, repeat=config.runner_repeat, min_repeat_ms=0,
                                      timeout=config.runner_timeout, enable_cpu_cache_flush=args.cold,
