@@ -109,3 +109,30 @@ def test_pretrained_model_from_shipped_records(hrn, tmp_path):
     finally:
         runner.close()
         builder.close()
+
+
+def test_attention_model_steers_a_search_on_the_gpu(hrn, tmp_path):
+    """The attention cost model, fitted on the shipped points of the other cases (CPU, a few seconds), steers the search of a
+    1024^3 fp16 GEMM on the real measurer; every measured kernel is verified."""
+    from heron_amd.pretrain import AttentionCostModel, RecordSet
+    data = RecordSet()
+    data.add_tree(os.path.join(os.path.dirname(os.path.abspath(__file__)), "pretrain", "records"))
+    model_path = str(tmp_path / "model.pt")
+    AttentionCostModel().fit(data, None, n_epoch=25, verbose=0).save(model_path)
+    env, task, runner, builder = _env(tmp_path, "CGA", 16, case=("gemm", [1024, 1024, 1024]), dtype=("float16", "float16"))
+    try:
+        env.config.pretrained_model = model_path
+        env.config.search_generations = 2
+
+        def ref(args):
+            A, Bm = workloads.gemm_f16_inputs(1024, 1024, 1024, seed=1)
+            return [A, Bm], oracle.gemm_f32(A, Bm)
+        task.set_verify_func(ref, rtol=1e-2)
+        env.tune("T1")
+        rows = [json.loads(l) for l in open(tmp_path / "OPS" / "T1" / "records.txt")]
+        assert 8 <= len(rows) <= 16 and all(row["perf"] > 0 for row in rows)
+        best = math.exp(-max(row["perf"] for row in rows))
+        assert 2.0 * 1024 ** 3 / best / 1e12 > 150
+    finally:
+        runner.close()
+        builder.close()
