@@ -144,6 +144,7 @@ SYMBOLS = {
     "hrn_probe_copy": (_i, [_vp, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_probe_launch": (_i, [_i, _i, ctypes.POINTER(_d), _vp]),
     "hrn_pad_rows": (_i, [_vp, _vp, ctypes.c_size_t, _i, _i, _i, _vp]),
+    "hrn_transpose_pad": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "hrn_probe_read": (_i, [_vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_last_error": (ctypes.c_char_p, []),
     "hrn_version": (ctypes.c_char_p, []),
@@ -244,6 +245,11 @@ def probe_launch(grid=256, repeat=2000, stream=0):
 def pad_rows(src_ptr, dst_ptr, rows, c, cp, elem_bytes, stream=0):
     """Zero-pads rows of c elements to cp elements (device pointers, dst holds rows * cp elements)."""
     _check(lib().hrn_pad_rows(src_ptr, dst_ptr, rows, c, cp, elem_bytes, stream))
+
+
+def transpose_pad(src_ptr, dst_ptr, batch, rows, cols, rows_padded, elem_bytes, stream=0):
+    """dst[b][c][r] = src[b][r][c], rows of dst zero-padded to rows_padded (device pointers)."""
+    _check(lib().hrn_transpose_pad(src_ptr, dst_ptr, batch, rows, cols, rows_padded, elem_bytes, stream))
 
 
 def probe_read(src_ptr, nbytes, repeat=10, stream=0):

@@ -644,6 +644,27 @@ __global__ void __launch_bounds__(256) pad_rows_kernel(const unsigned char* __re
     }
 }
 
+// Batched transpose src[b][r][c] -> dst[b][c][r'] with r' padded to rp >= rows (zeros), through a 64x64 LDS tile so that
+// both the reads (along c) and the writes (along r) are contiguous.  blockDim = (64, 4).
+template <typename T>
+__global__ void __launch_bounds__(256) transpose_pad_kernel(const T* __restrict__ src, T* __restrict__ dst,
+                                                            int rows, int cols, int rp) {
+    __shared__ T tile[64][65];
+    const size_t b = blockIdx.z;
+    const T* in = src + b * (size_t)rows * cols;
+    T* out = dst + b * (size_t)cols * rp;
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    for (int i = threadIdx.y; i < 64; i += 4) {
+        const int r = r0 + i, c = c0 + threadIdx.x;
+        tile[i][threadIdx.x] = (r < rows && c < cols) ? in[(size_t)r * cols + c] : (T)0;
+    }
+    __syncthreads();
+    for (int i = threadIdx.y; i < 64; i += 4) {
+        const int c = c0 + i, r = r0 + threadIdx.x;
+        if (c < cols && r < rp) out[(size_t)c * rp + r] = tile[threadIdx.x][i];
+    }
+}
+
 // streams `n16` 16-byte words through every lane without storing anything: the read-only counterpart of the copy probe
 __global__ void __launch_bounds__(256) probe_read_kernel(const pv4i* __restrict__ src, size_t n16) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -677,6 +698,22 @@ int hrn_pad_rows(const void* src, void* dst, size_t rows, int c, int cp, int ele
     else pad_rows_kernel<1><<<grid, 256, 0, st>>>((const unsigned char*)src, (unsigned char*)dst, rows, c, cp);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HRN_E_LAUNCH, "pad_rows: %s", hipGetErrorString(e));
+    return HRN_OK;
+}
+
+int hrn_transpose_pad(const void* src, void* dst, int batch, int rows, int cols, int rows_padded, int elem_bytes, void* stream) {
+    if (!src || !dst || batch < 0 || rows < 1 || cols < 1 || rows_padded < rows || batch > 65535 ||
+        (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4))
+        return fail(HRN_E_BADPARAM, "transpose_pad: batch %d, %d x %d -> %d x %d, %d-byte elements", batch, rows, cols, cols, rows_padded, elem_bytes);
+    if (batch == 0) return HRN_OK;
+    const dim3 grid((cols + 63) / 64, (rows_padded + 63) / 64, batch), block(64, 4);
+    if (grid.y > 65535) return fail(HRN_E_BADPARAM, "transpose_pad: %d rows are more than 65535 tiles", rows_padded);
+    hipStream_t st = (hipStream_t)stream;
+    if (elem_bytes == 1) transpose_pad_kernel<unsigned char><<<grid, block, 0, st>>>((const unsigned char*)src, (unsigned char*)dst, rows, cols, rows_padded);
+    else if (elem_bytes == 2) transpose_pad_kernel<unsigned short><<<grid, block, 0, st>>>((const unsigned short*)src, (unsigned short*)dst, rows, cols, rows_padded);
+    else transpose_pad_kernel<unsigned int><<<grid, block, 0, st>>>((const unsigned int*)src, (unsigned int*)dst, rows, cols, rows_padded);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HRN_E_LAUNCH, "transpose_pad: %s", hipGetErrorString(e));
     return HRN_OK;
 }
 

@@ -80,6 +80,31 @@ def _pad_last(t, to):
     return torch.nn.functional.pad(t, (0, to - c)).contiguous()
 
 
+def _native_ok(t):
+    return t.is_cuda and t.is_contiguous() and t.element_size() in (1, 2, 4)
+
+
+def _channels_last(x3, cp=None):
+    """(N, C, L) -> (N, L, cp): channels become the last axis, zero-padded to ``cp`` (one pass of the library)."""
+    N, C, L = x3.shape
+    cp = cp or C
+    if _native_ok(x3) and N <= 65535 and L > 0:
+        out = torch.empty((N, L, cp), dtype=x3.dtype, device=x3.device)
+        B.transpose_pad(x3.data_ptr(), out.data_ptr(), N, C, L, cp, x3.element_size(), _stream())
+        return out
+    return _pad_last(x3.permute(0, 2, 1), cp)
+
+
+def _channels_first(y3):
+    """(N, L, C) -> (N, C, L)."""
+    N, L, C = y3.shape
+    if _native_ok(y3) and N <= 65535 and L > 0:
+        out = torch.empty((N, C, L), dtype=y3.dtype, device=y3.device)
+        B.transpose_pad(y3.data_ptr(), out.data_ptr(), N, L, C, L, y3.element_size(), _stream())
+        return out
+    return y3.permute(0, 2, 1).contiguous()
+
+
 # Every adapter has two halves: ``act`` maps the activation input(s) to the kernel's A operand and is needed on every
 # call; ``const`` maps the constant input (filter, vector) - or nothing but the shapes - to the kernel's B operand and is
 # needed once per set of weights (run_operator caches it when asked to).
@@ -142,7 +167,7 @@ def _const_c1d_nwc(info, X, F):           # (K,CI,CO)
 
 
 def _act_c1d_ncw(info, X, F):             # (N,CI,W)
-    return _pad_last(X.permute(0, 2, 1), _cpad(info)).unsqueeze(1)
+    return _channels_last(X, _cpad(info)).unsqueeze(1)
 
 
 def _const_c1d_ncw(info, X, F):           # (CO,CI,KW)
@@ -150,7 +175,8 @@ def _const_c1d_ncw(info, X, F):           # (CO,CI,KW)
 
 
 def _act_nchw(info, X, F):                # (N,CI,H,W)
-    return _pad_last(X.permute(0, 2, 3, 1), _cpad(info))
+    N, CI, H, W = X.shape
+    return _channels_last(X.reshape(N, CI, H * W), _cpad(info)).reshape(N, H, W, _cpad(info))
 
 
 def _const_oihw(info, X, F):              # (CO,CI,KH,KW)
@@ -189,7 +215,8 @@ def _const_c3d_dhwio(info, X, F):         # (KD,KH,KW,CI,CO)
 
 
 def _act_c3d_ncdhw(info, X, F):           # (N,CI,D,H,W)
-    return _act_c3d_ndhwc(info, X.permute(0, 2, 3, 4, 1), F)
+    N, CI, D, H, W = X.shape
+    return _act_c3d_ndhwc(info, _channels_last(X.reshape(N, CI, D * H * W)).reshape(N, D, H, W, CI), F)
 
 
 def _const_c3d_oidhw(info, X, F):         # (CO,CI,KD,KH,KW)
@@ -243,11 +270,12 @@ def _fin_c1d_nwc(info, C):                # (N,1,WO,CO) -> (N,WO,CO)
 
 
 def _fin_c1d_ncw(info, C):                # -> (N,CO,WO)
-    return C.squeeze(1).permute(0, 2, 1).contiguous()
+    return _channels_first(C.squeeze(1))
 
 
 def _fin_nchw(info, C):                   # (N,HO,WO,CO) -> (N,CO,HO,WO)
-    return C.permute(0, 3, 1, 2).contiguous()
+    N, HO, WO, CO = C.shape
+    return _channels_first(C.reshape(N, HO * WO, CO)).reshape(N, CO, HO, WO)
 
 
 def _fin_c3d_ndhwc(info, C):              # (N*DO,HO,WO,CO) -> (N,DO,HO,WO,CO)
@@ -256,7 +284,9 @@ def _fin_c3d_ndhwc(info, C):              # (N*DO,HO,WO,CO) -> (N,DO,HO,WO,CO)
 
 
 def _fin_c3d_ncdhw(info, C):              # -> (N,CO,DO,HO,WO)
-    return _fin_c3d_ndhwc(info, C).permute(0, 4, 1, 2, 3).contiguous()
+    Y = _fin_c3d_ndhwc(info, C)
+    N, DO, HO, WO, CO = Y.shape
+    return _channels_first(Y.reshape(N, DO * HO * WO, CO)).reshape(N, CO, DO, HO, WO)
 
 
 ADAPTERS = {

@@ -226,6 +226,15 @@ int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, co
 int hrn_pad_rows(const void* src, void* dst, size_t rows, int c, int cp, int elem_bytes, void* stream);
 
 /*
+ * Layout pre-stage / post-stage: batched transpose src[batch][rows][cols] -> dst[batch][cols][rows_padded], the tail of
+ * every output row (rows..rows_padded) zero-filled; elements of 1, 2 or 4 bytes.  Channels-first activations
+ * (N,C,H*W) become channels-last with padded channels in one pass, and a channels-last result goes back to
+ * channels-first: the layout stages the reference inlines around its tensorized product for the NCHW / NCW
+ * operators (ops/cuda/conv2d.py:9-135, ops/cuda/conv1d.py).  Both buffers are caller-owned device memory.
+ */
+int hrn_transpose_pad(const void* src, void* dst, int batch, int rows, int cols, int rows_padded, int elem_bytes, void* stream);
+
+/*
  * Roofline probes (no counterpart in the reference, which never relates a timing to a hardware
  * limit).  hrn_probe_mfma times a register-resident loop of independent MFMAs of the given
  * dtype/shape on every CU and returns dense T(FL)OP/s (random_operands != 0 feeds operands with the

@@ -203,3 +203,27 @@ def test_pad_rows_kernel(hrn):
     assert torch.equal(hostops._pad_last(x, 8), torch.nn.functional.pad(x, (0, 5)))
     with pytest.raises(B.HeronRocmError):
         B.pad_rows(x.data_ptr(), x.data_ptr(), 4, 3, 6, 2, 0)            # 12-byte rows are not whole 16-byte words
+
+
+def test_transpose_pad_kernel(hrn):
+    """The layout pre-/post-stage of the library against torch: three element sizes, sizes off the 64x64 tile, padding."""
+    import torch
+    st = torch.cuda.current_stream().cuda_stream
+    for dtype in (torch.float16, torch.uint8, torch.int32):
+        for (b, r, c, rp) in [(1, 3, 50, 8), (2, 64, 64, 64), (3, 65, 129, 72), (2, 20, 1000, 24), (1, 1, 1, 1), (4, 130, 7, 130)]:
+            if dtype == torch.float16:
+                x = torch.randn((b, r, c), device="cuda").to(dtype)
+            else:
+                x = torch.randint(0, 120, (b, r, c), device="cuda").to(dtype)
+            out = torch.full((b, c, rp), 9, dtype=dtype, device="cuda")
+            B.transpose_pad(x.data_ptr(), out.data_ptr(), b, r, c, rp, x.element_size(), st)
+            torch.cuda.synchronize()
+            ref = torch.nn.functional.pad(x.permute(0, 2, 1), (0, rp - r)).contiguous()
+            assert torch.equal(out, ref), (dtype, b, r, c, rp)
+    x = torch.randn((2, 5, 33), device="cuda").half()
+    assert torch.equal(hostops._channels_last(x, 8), torch.nn.functional.pad(x.permute(0, 2, 1), (0, 3)))
+    assert torch.equal(hostops._channels_first(x), x.permute(0, 2, 1).contiguous())
+    with pytest.raises(B.HeronRocmError):
+        B.transpose_pad(x.data_ptr(), x.data_ptr(), 1, 8, 8, 4, 2, st)             # padded rows fewer than rows
+    with pytest.raises(B.HeronRocmError):
+        B.transpose_pad(x.data_ptr(), x.data_ptr(), 1, 8, 8, 8, 3, st)             # 3-byte elements
