@@ -433,7 +433,7 @@ def test_refinement_rounds_measure_one_knob_neighbours(tmp_path, capsys):
     for s in near:
         vals = s.knob_manager.solved_knob_vals_phenotype
         assert s.valid and solver.SATScore(vals) == 0
-        assert min(sum(1 for n in names if vals[n] != top[n]) for top in tops) == 1
+        assert 1 in [sum(1 for n in names if vals[n] != top[n]) for top in tops]      # (it may coincide with the other incumbent)
     # the share is a config key read at run time; 0 gives the plain loop, and so does any tuner but the constrained GA
     env.config.refine_share = 0
     assert t.refinement_share() == 0.0
