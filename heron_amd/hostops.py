@@ -231,7 +231,13 @@ def _act_t2d_nchw(info, X, F):            # (N,CI,H,W): zero-expanded by the str
     top = (c['KH'] - 1) * t['dil'] - t['pad']
     left = (c['KW'] - 1) * t['dil'] - t['pad']
     Xe = torch.zeros((N, c['H'], c['W'], c['CI']), dtype=X.dtype, device=X.device)
-    Xe[:, top: top + (H - 1) * s + 1: s, left: left + (W - 1) * s + 1: s, :CI] = X.permute(0, 2, 3, 1)
+    if s > 1:
+        # channels last (and padded) first, so that the strided scatter moves whole pixels (stride 2: 137 -> 70 us end
+        # to end on 16x56x56x64); with stride 1 the permuted assignment is one pass and an extra launch only costs
+        Xe[:, top: top + (H - 1) * s + 1: s, left: left + (W - 1) * s + 1: s, :] = \
+            _channels_last(X.reshape(N, CI, H * W), c['CI']).reshape(N, H, W, c['CI'])
+    else:
+        Xe[:, top: top + H, left: left + W, :CI] = X.permute(0, 2, 3, 1)
     return Xe
 
 
