@@ -154,21 +154,29 @@ class Tuner:
         """Feasible points that differ from one of the ``top`` best measured points in exactly one knob (the solver
         re-derives the dependent variables), scored by the cost model."""
         out, seen = [], set()
+
+        def consider(knobs):
+            s = Sample(env.task)
+            point, valid = s.knob_manager.validate(knobs)
+            code = Code(point) if valid else None
+            if valid and code not in seen:
+                seen.add(code)
+                s.point, s.valid, s.stmt_code, s.violation = point, True, code, 0
+                out.append(s)
+
         for base in reversed(self.history_topk_samples(env, top)):
             geno = base.knob_manager.solved_knob_vals_genotype
             names = base.knob_manager.knob_names
             for name in names:
                 for cand in base.knob_manager.get_knob_candidates(name):
-                    if cand == geno[name]:
-                        continue
-                    s = Sample(env.task)
-                    point, valid = s.knob_manager.validate({n: (cand if n == name else geno[n]) for n in names})
-                    code = Code(point) if valid else None
-                    if not valid or code in seen:
-                        continue
-                    seen.add(code)
-                    s.point, s.valid, s.stmt_code, s.violation = point, True, code, 0
-                    out.append(s)
+                    if cand != geno[name]:
+                        consider({n: (cand if n == name else geno[n]) for n in names})
+            # one coupled move that no single knob reaches: the same block tile with the wave grid transposed
+            # (knobs named ..._m / ..._n in pairs swap their values)
+            twin = {n: n[:-2] + ("_n" if n.endswith("_m") else "_m") for n in names if n.endswith(("_m", "_n"))}
+            twin = {n: t for n, t in twin.items() if t in geno and not n.endswith("group_m")}
+            if twin:
+                consider({n: geno[twin.get(n, n)] for n in names})
         return self._assign_predictions(out)
 
     # ------------------------------------------------------------------------------------------------ feasibility table
