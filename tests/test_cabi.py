@@ -114,3 +114,23 @@ def test_compile_error_paths(tmp_path, monkeypatch):
     monkeypatch.setenv("HRN_HIPCC", str(slow))
     assert L.hrn_compile(ctypes.byref(d), 0.5, buf, 4096) == -5 and b"exceeded" in L.hrn_last_error()
     assert not list((tmp_path / "cache").glob("*.hsaco"))
+
+
+def test_prestage_entry_points_reject_bad_arguments_without_a_gpu():
+    """Argument checks of the pre-stage kernels and probes run before any HIP call, so they can be exercised here."""
+    L = B.lib()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert L.hrn_pad_rows(p, p, 4, 3, 6, 2, None) == B.HRN_E_BADPARAM          # 12-byte rows are not whole 16-byte words
+    assert b"pad_rows" in L.hrn_last_error()
+    assert L.hrn_pad_rows(p, p, 4, 9, 8, 2, None) == B.HRN_E_BADPARAM          # padded row shorter than the row
+    assert L.hrn_pad_rows(None, p, 4, 3, 8, 2, None) == B.HRN_E_BADPARAM
+    assert L.hrn_pad_rows(p, p, 0, 3, 8, 2, None) == 0                          # nothing to do is not an error
+    assert L.hrn_transpose_pad(p, p, 1, 8, 8, 4, 2, None) == B.HRN_E_BADPARAM   # fewer padded rows than rows
+    assert L.hrn_transpose_pad(p, p, 1, 8, 8, 8, 3, None) == B.HRN_E_BADPARAM   # 3-byte elements
+    assert L.hrn_transpose_pad(p, p, 70000, 8, 8, 8, 2, None) == B.HRN_E_BADPARAM
+    assert L.hrn_transpose_pad(p, p, 0, 8, 8, 8, 2, None) == 0
+    out = ctypes.c_double()
+    assert L.hrn_probe_launch(0, 10, ctypes.byref(out), None) == B.HRN_E_BADPARAM
+    assert L.hrn_probe_launch(256, 10, None, None) == B.HRN_E_BADPARAM
+    assert L.hrn_probe_read(p, 24, 1, ctypes.byref(out), None) == B.HRN_E_BADPARAM   # not a multiple of 16 bytes
