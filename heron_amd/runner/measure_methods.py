@@ -113,39 +113,68 @@ LocalBuilder = HipBuilder
 _TORCH_DT = {"float16": "float16", "uint8": "uint8", "int8": "int8", "int32": "int32"}
 
 
-def _time_operator(torch, mod, info, prob, number, repeat, min_repeat_ms):
-    """Seconds per call of hostops.run_operator, time_evaluator style: activation pre-stage + kernel + result reorder.
-    The constant operand (reordered filter, generated right-hand side) is prepared once outside the timed calls, as a
-    caller with fixed weights does."""
-    from .. import hostops
+def _operator_inputs(torch, info, ref_input):
+    """Device tensors in the operator's own layouts: the reference inputs when given, random data otherwise.  The
+    shapes must be the ones the operator declares (a mismatch would let the kernel read past an allocation)."""
     f16 = info['kind'] == 'f16'
     names = [n for n in info['reference_args'] if n != 'out']
+    shapes = [tuple(int(x) for x in info['reference_args'][n]) for n in names]
+    if ref_input is not None:                      # every shape is checked before anything is uploaded
+        if len(ref_input) < len(names):
+            raise ValueError("reference inputs: %d given, operator takes %d" % (len(ref_input), len(names)))
+        for i, shape in enumerate(shapes):
+            if tuple(np.shape(ref_input[i])) != shape:
+                raise ValueError("reference input %d has shape %s, the operator declares %s"
+                                 % (i, tuple(np.shape(ref_input[i])), shape))
     inputs = []
-    for i, n in enumerate(names):
-        shape = tuple(info['reference_args'][n])
-        if f16:
+    for i, shape in enumerate(shapes):
+        want = torch.float16 if f16 else (torch.uint8 if i == 0 else torch.int8)
+        if ref_input is not None:
+            t = torch.from_numpy(np.ascontiguousarray(ref_input[i])).to(want).cuda()
+        elif f16:
             t = (torch.rand(shape, device="cuda") * 2 - 1).half()
         elif i == 0:
             t = torch.randint(0, 256, shape, dtype=torch.uint8, device="cuda")
         else:
             t = torch.randint(-128, 128, shape, dtype=torch.int8, device="cuda")
         inputs.append(t)
+    return inputs
+
+
+def _time_operator(torch, mod, info, prob, number, repeat, min_repeat_ms, ref_input=None, flush=None):
+    """(seconds per call, result of the last call) of hostops.run_operator, time_evaluator style: activation pre-stage +
+    kernel + result reorder - the same definition with and without a result check.  The constant operand (reordered
+    filter, generated right-hand side) is prepared once outside the timed calls, as a caller with fixed weights does.
+    With ``flush`` (a device buffer larger than the caches) every repeat is ONE call after the buffer was streamed
+    through the caches."""
+    from .. import hostops
+    inputs = _operator_inputs(torch, info, ref_input)
     gm, sk = int(prob.get('group_m', 8)), int(prob.get('split_k', 0))
     weights = hostops.prepare_constant(info, inputs)
 
     def call():
         return hostops.run_operator(mod, info, inputs, group_m=gm, split_k=sk, constant=weights)
 
-    call()                                                                   # warm-up, surfaces launch errors
+    out = call()                                                             # warm-up, surfaces launch errors
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     costs = []
+    if flush is not None:
+        half = flush.numel() // 2
+        for _ in range(repeat):
+            flush[half:2 * half].copy_(flush[:half])
+            e0.record()
+            out = call()
+            e1.record()
+            e1.synchronize()
+            costs.append(e0.elapsed_time(e1) * 1e-3)
+        return costs, out
     for _ in range(repeat):
         num = number
         while True:
             e0.record()
             for _i in range(num):
-                call()
+                out = call()
             e1.record()
             e1.synchronize()
             ms = e0.elapsed_time(e1)
@@ -154,7 +183,14 @@ def _time_operator(torch, mod, info, prob, number, repeat, min_repeat_ms):
                 number = num
                 break
             num = max(num + 1, int(min(65536.0, min_repeat_ms * 1.2 / max(ms / num, 1e-4) + 1)))
-    return costs
+    return costs, out
+
+
+def _matches(ref_output, out, rtol):
+    ref = np.asarray(ref_output, dtype=np.float64)
+    if tuple(ref.shape) != tuple(out.shape):
+        return False
+    return bool(np.allclose(ref, out.astype(np.float64), rtol=rtol, atol=rtol * float(np.abs(ref).max()) * 1e-2))
 
 
 def _server_main(conn, device_id):
@@ -192,17 +228,28 @@ def _server_main(conn, device_id):
             p = B.Problem()
             for k, v in prob.items():
                 setattr(p, k, v)
-            if adapter is not None and ref_input is None:
+            if cold and flush is None:
+                flush = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+            if adapter is not None:
                 # the operator reaches the kernel through an operand adapter: time pre-stage + kernel + post-stage on
-                # operands in the operator's own layouts, so that the record's latency is what a caller pays
-                costs = _time_operator(torch, mod, adapter, prob, number, repeat, min_repeat_ms)
-                conn.send(("ok", (costs, MeasureErrorNo.NO_ERROR)))
+                # operands in the operator's own layouts (the reference inputs when the result is checked), so that
+                # the record's latency is what a caller pays and the kernel never sees an operand of the wrong size
+                costs, out = _time_operator(torch, mod, adapter, prob, number, repeat, min_repeat_ms, ref_input,
+                                            flush if cold else None)
+                errno = MeasureErrorNo.NO_ERROR
+                if ref_output is not None and not _matches(ref_output, out.cpu().numpy(), rtol):
+                    errno = MeasureErrorNo.VERIFY_FAILED
+                conn.send(("ok", (costs, errno)))
                 continue
             tensors = []
             for i, (shape, dtype) in enumerate(arg_info):
                 tdt = getattr(torch, _TORCH_DT[dtype])
                 if ref_input is not None and i < len(ref_input):
-                    t = torch.from_numpy(np.ascontiguousarray(ref_input[i])).cuda()
+                    host = np.ascontiguousarray(ref_input[i])
+                    if tuple(host.shape) != tuple(shape):
+                        raise ValueError("reference input %d has shape %s, the kernel's operand is %s"
+                                         % (i, tuple(host.shape), tuple(shape)))
+                    t = torch.from_numpy(host).to(tdt).cuda()
                 elif i == len(arg_info) - 1:
                     t = torch.empty(shape, dtype=tdt, device="cuda")
                 elif dtype == "float16":
@@ -215,8 +262,6 @@ def _server_main(conn, device_id):
             torch.cuda.synchronize()
             if cold:
                 # every launch starts from flushed caches (the reference runner's enable_cpu_cache_flush, on the GPU)
-                if flush is None:
-                    flush = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
                 costs = mod.time_cold(p, tensors[0].data_ptr(), tensors[1].data_ptr(), tensors[-1].data_ptr(),
                                       flush.data_ptr(), flush.numel(), repeat, 0)
             else:
@@ -224,9 +269,7 @@ def _server_main(conn, device_id):
                                  number, repeat, min_repeat_ms, 0)
             errno = MeasureErrorNo.NO_ERROR
             if ref_output is not None:
-                out = tensors[-1].cpu().numpy()
-                if not np.allclose(np.asarray(ref_output, dtype=np.float64), out.astype(np.float64), rtol=rtol,
-                                   atol=rtol * float(np.abs(ref_output).max()) * 1e-2):
+                if not _matches(ref_output, tensors[-1].cpu().numpy(), rtol):
                     errno = MeasureErrorNo.VERIFY_FAILED
             conn.send(("ok", (costs, errno)))
         except Exception as e:  # noqa: BLE001 - reported to the tuning process

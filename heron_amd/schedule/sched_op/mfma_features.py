@@ -64,14 +64,17 @@ def analytic_seconds(info, v):
     t_lds = frag_bytes * lds_conflict_ways(bkb, v['lds_swizzle']) / (256 * 2.1e9)
     parts = sorted((t_mfma, t_fetch, t_lds))
     k_tiles = max(1, math.ceil(kbytes / bkb))
-    hidden = min(per_cu, on_busiest_cu)
     sync = k_tiles * BARRIER * (1.0 + waves / 16.0) * (0.6 if v['lds_stages'] > 2 else 1.0)
-    t_wg = parts[2] + 0.35 * parts[1] + 0.1 * parts[0] + sync + WG_FIXED / hidden      # the three overlap only partly
+    # Throughput work (matrix pipe, fetch path, LDS: shared by the workgroups of a CU) adds up over all the CU's
+    # workgroups; waiting (barriers, start-up and drain of a workgroup) is paid once per round of co-resident ones.
+    t_busy = parts[2] + 0.35 * parts[1] + 0.1 * parts[0]                                # the three overlap only partly
+    t_wait = sync + WG_FIXED
+    rounds = math.ceil(on_busiest_cu / per_cu)
     out_bytes = 2 if info['kind'] == 'f16' else 4
     moved = g['batch'] * (g['M'] * g['K'] * es + g['N'] * g['K'] * es + g['M'] * g['N'] * out_bytes)
     if split > 1:
         moved += 2 * split * g['batch'] * g['M'] * g['N'] * 4      # partial sums written and read back
-    return max(on_busiest_cu * t_wg / min(per_cu, on_busiest_cu) * min(per_cu, on_busiest_cu), moved / HBM) + LAUNCH * (2 if split > 1 else 1)
+    return max(on_busiest_cu * t_busy + rounds * t_wait, moved / HBM) + LAUNCH * (2 if split > 1 else 1)
 
 
 def featurize(info, values):

@@ -442,3 +442,57 @@ def test_refinement_rounds_measure_one_knob_neighbours(tmp_path, capsys):
     assert t.refinement_share() == 0.0
     from heron_amd.tuner.random_tuner import CRandTuner
     assert CRandTuner(env.config).refinement_share() == 0.0
+
+
+def test_stem_reference_inputs_match_the_operator_not_the_padded_kernel():
+    """--check on a 3-channel stem: the host reference yields unpadded (N,H,W,3) / (CO,KH,KW,3) arrays while the kernel
+    runs on 8 padded channels.  The measurer must take them through the operand adapter (operator layouts), and must
+    refuse operands whose shapes differ from what the operator declares."""
+    import importlib.util
+    from heron_amd.runner import measure_methods as MM
+    spec = importlib.util.spec_from_file_location(
+        "rocm_run", os.path.join(os.path.dirname(__file__), "quick_start", "rocm", "run.py"))
+    run_py = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(run_py)
+
+    class Ctx:
+        def set_info(self, info):
+            self.info = info
+
+        def set_axis_map(self, m):
+            pass
+
+    params = [2, 20, 20, 3, 16, 7, 7, 2, 3, 1, "float16", "float16"]
+    ctx = Ctx()
+    outs = getOpFromName("c2d")(ctx, *params)
+    info = ctx.info
+    assert info['adapter'] == 'c2d_krsc' and info['conv']['CI'] == 8
+    kernel_shapes = [tuple(t.shape) for t in outs[0].op.input_tensors]
+    assert kernel_shapes == [(2, 20, 20, 8), (16, 7, 7, 8)]
+    ref_input, ref_output = run_py.host_reference("c2d")(params)
+    declared = [tuple(v) for k, v in info['reference_args'].items() if k != 'out']
+    assert [tuple(x.shape) for x in ref_input] == declared == [(2, 20, 20, 3), (16, 7, 7, 3)]
+    assert tuple(ref_output.shape) == tuple(outs[0].shape)
+
+    class NoCuda:                       # stands in for torch: reaching the upload would be the bug
+        float16 = uint8 = int8 = None
+
+    with pytest.raises(ValueError, match="declares"):
+        MM._operator_inputs(NoCuda, info, [np.zeros(kernel_shapes[0], np.float16), ref_input[1]])
+    with pytest.raises(ValueError, match="operator takes"):
+        MM._operator_inputs(NoCuda, info, [ref_input[0]])
+
+
+def test_analytic_estimate_rewards_co_resident_workgroups():
+    """Two points that differ only in how many workgroups fit a CU side by side (LDS of one workgroup): the waiting
+    parts of the estimate are paid once per round of co-resident workgroups, so the roomier point must be faster."""
+    from heron_amd.schedule.sched_op.mfma_features import analytic_seconds
+    info = {'kind': 'f16', 'gemm_view': dict(batch=192, M=512, N=512, K=64)}
+    v = dict(mfma=16, wave_m=2, wave_n=2, tile_m=4, tile_n=4, block_k_bytes=128, conv_window=0, persistent=0,
+             lds_stages=2, lds_swizzle=2, waves_per_eu=0, epilogue=1, split_k=1, raster_group_m=4, issue_order=1,
+             load_spread=2, block_m=128, block_n=128, waves=4, k_steps=2, k_tiles=1, grid_m=4, grid_n=4,
+             lds_bytes=65536, window_bytes=0, regs_per_lane=120, loads_per_tile=8)
+    two_per_cu = analytic_seconds(info, v)
+    one_per_cu = analytic_seconds(info, dict(v, lds_bytes=120000))
+    four_per_cu = analytic_seconds(info, dict(v, lds_bytes=32768))
+    assert four_per_cu <= two_per_cu < one_per_cu        # (two per CU already reach the HBM floor of this shape)
