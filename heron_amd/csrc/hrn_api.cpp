@@ -39,6 +39,7 @@ struct HrnKArgs {  // must match mfma_gemm_template.hip
     int32_t H, W, CI, HO, WO, KH, KW, cstride, cpad, cdil;
     int32_t cstride_w, cpad_w, cdil_w;
     int32_t split, kt_per_slice;
+    const void* bsum;
 };
 
 struct hrn_module {
@@ -135,7 +136,7 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (d->stages < 2 || d->stages > 5) return fail(HRN_E_BADPARAM, "stages %d not in 2..5", d->stages);
     if (d->swizzle < 0 || d->swizzle > 3) return fail(HRN_E_BADPARAM, "swizzle %d", d->swizzle);
     if (d->epilogue < 0 || d->epilogue > 2) return fail(HRN_E_BADPARAM, "epilogue %d", d->epilogue);
-    if (d->sched < 0 || d->sched > 1) return fail(HRN_E_BADPARAM, "sched %d", d->sched);
+    if (d->sched < 0 || d->sched > 2) return fail(HRN_E_BADPARAM, "sched %d", d->sched);
     if (d->load_spread < 0 || d->load_spread > 3) return fail(HRN_E_BADPARAM, "load_spread %d", d->load_spread);
     if (d->waves_per_eu < 0 || d->waves_per_eu > 8) return fail(HRN_E_BADPARAM, "waves_per_eu %d", d->waves_per_eu);
     if (d->conv_window < 0 || d->conv_window > 1) return fail(HRN_E_BADPARAM, "conv_window %d", d->conv_window);
@@ -145,6 +146,8 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (d->persistent && (d->epilogue < 1 || d->conv_window || d->split_k))
         return fail(HRN_E_BADPARAM, "persistent needs the LDS-staged epilogue and neither conv_window nor split_k");
     if (d->split_k && d->conv_window) return fail(HRN_E_BADPARAM, "split_k uses the im2col load path, not conv_window");
+    if (d->sched == 2 && (d->wm * d->wn != 8 || d->conv_window || d->persistent || d->split_k))
+        return fail(HRN_E_BADPARAM, "sched 2 (two wave groups) needs 8 waves and neither conv_window, persistent nor split_k");
     Derived r;
     r.es = d->dtype == HRN_DT_F16 ? 2 : 1;
     r.oes = (d->dtype == HRN_DT_F16 && !d->split_k) ? 2 : 4;

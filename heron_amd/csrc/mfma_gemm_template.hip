@@ -47,6 +47,7 @@ struct HrnKArgs {
     int32_t H, W, CI, HO, WO, KH, KW, cstride, cpad, cdil;
     int32_t cstride_w, cpad_w, cdil_w;   // conv: the width-direction values (cstride/cpad/cdil are the height ones)
     int32_t split, kt_per_slice;         // split-K: number of K slices and k-tiles per slice
+    const void* bsum;                    // uint8 path: per batch entry N column sums of B (sum_k B[n,k], int32), or null
 };
 #endif
 
@@ -57,18 +58,6 @@ constexpr int OP = HRN_OP;
 constexpr int BM = HRN_BM, BN = HRN_BN, BKB = HRN_BKB;
 constexpr int WM = HRN_WM, WN = HRN_WN, MT = HRN_MFMA, NS = HRN_STAGES, SWZ = HRN_SWZ;
 constexpr int EPI = HRN_EPI;
-// Study switches for bottleneck analysis, set only through extra compiler flags (results are WRONG when non-zero):
-// 1 skip LDS fragment reads after the first tile, 2 skip global->LDS loads after the prologue, 4 drop the per-tile
-// barrier, 8 skip the MFMAs, 16 skip the stores of C.
-#ifndef HRN_ABLATE
-#define HRN_ABLATE 0
-#endif
-constexpr int ABL = HRN_ABLATE;
-// timing study only (results are wrong): keep HRN_FAKE_DEPTH k-tiles in flight, written round-robin over the NS stages
-#ifndef HRN_FAKE_DEPTH
-#define HRN_FAKE_DEPTH 0
-#endif
-constexpr int FD = HRN_FAKE_DEPTH;
 // Conv window mode (HRN_OP=1, stride 1, dilation 1, 'same' padding): instead of fetching an im2col tile of A for every
 // filter tap, the workgroup loads ONCE the window of input pixels its BM output pixels can reach (a contiguous range
 // of BM + 2*(pad_h*W + pad_w) pixels, all channels) and every tap reads its operand fragments from that window at a row offset
@@ -95,7 +84,8 @@ constexpr bool PERS = (HRN_PERSIST != 0);
 #endif
 constexpr bool SPLITK = (HRN_SPLITK != 0);
 // Issue order of a k-step: 1 = the source order of the row groups is pinned (a scheduling fence after every row of
-// MFMAs), 0 = the compiler interleaves on its own, guided by group hints (one LDS read per few MFMAs).
+// MFMAs), 0 = the compiler interleaves on its own, guided by group hints (one LDS read per few MFMAs), 2 = the two
+// wave groups of an 8-wave workgroup alternate between a memory phase and a matrix phase (see "SCHED 2" below).
 #ifndef HRN_SCHED
 #define HRN_SCHED 1
 #endif
@@ -145,13 +135,13 @@ constexpr int LDS_BYTES = PERS ? NS * STAGE_BYTES + EPI_BYTES
                                : ((CW || NS * STAGE_BYTES > EPI_BYTES) ? NS * STAGE_BYTES : EPI_BYTES);
 constexpr int STORES_PER_TILE = (EPI >= 1) ? TM * ESPLIT * (MT * (SW * OES / 16) / 64) : 0;   // store instructions per wave per output tile
 static_assert(EPI >= 0 && EPI <= 2 && TN % ESPLIT == 0, "epilogue kind");
-static_assert(!PERS || (EPI >= 1 && !CW && !SPLITK && HRN_ABLATE == 0 && KS % 2 == 0), "persistent mode: staged epilogue, even k-steps");
+static_assert(!PERS || (EPI >= 1 && !CW && !SPLITK && KS % 2 == 0), "persistent mode: staged epilogue, even k-steps");
 static_assert(!PERS || (NS - 2) * LPT + STORES_PER_TILE <= 63, "persistent mode: vmcnt range");
 static_assert(!SPLITK || !CW, "split-K uses the im2col load path");
 static_assert(LDS_BYTES <= 163840, "LDS");
 static_assert(EPI == 0 || (MT * (SW * OES / 16)) % 64 == 0, "staged epilogue: a strip must split into whole wave stores");
 static_assert(SWZ == 0 || (CPR << (SWZ - 1)) <= MT, "swizzle period must fit in one MFMA tile");
-static_assert(((FD ? FD : NS) - 1) * LPT <= 63, "vmcnt range");
+static_assert((NS - 1) * LPT <= 63, "vmcnt range");
 static_assert(NT <= 1024, "threads");
 static_assert(DT == 0 || NS * STAGE_BYTES >= WM * BN * 4, "column sums must fit the stages");
 
@@ -213,6 +203,24 @@ __device__ __forceinline__ v4i mfma(v4i x, v4i y, v4i c) {
     return __builtin_amdgcn_mfma_i32_16x16x64_i8(x, y, c, 0, 0, 0);
 }
 
+// In-place form for the two-group schedule: the accumulator is both source and destination, so its registers stay
+// where they are for the whole k-loop (with the intrinsic the register allocator is free to move them from step to
+// step, and with the single fragment buffer of that schedule it does, at the price of spills).  The compiler does not
+// know this instruction's latency: code that reads the accumulators afterwards starts with mfma_drain().
+__device__ __forceinline__ void mfma_inplace(v4i x, v4i y, v16f& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(x), "v"(y));
+}
+__device__ __forceinline__ void mfma_inplace(v4i x, v4i y, v4f& c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(x), "v"(y));
+}
+__device__ __forceinline__ void mfma_inplace(v4i x, v4i y, v16i& c) {
+    asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(c) : "v"(x), "v"(y));
+}
+__device__ __forceinline__ void mfma_inplace(v4i x, v4i y, v4i& c) {
+    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(c) : "v"(x), "v"(y));
+}
+__device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+
 // Scheduling hints of one k-step (HRN_SCHED = 0): NR groups of {1 LDS read, NV/NR buffer loads, NMM/NR MFMAs}.
 template <int R, int NR, int NMM, int NV>
 __device__ __forceinline__ void sched_hint() {
@@ -260,8 +268,11 @@ hrn_mfma_kernel(const HrnKArgs a) {
         const int first_m = gid * a.group_m;
         const int gsz = min(a.tiles_m - first_m, a.group_m);
         const int tin = t - gid * group_sz;
-        tile_m = first_m + tin % gsz;
-        tile_n = tin / gsz;
+        // (the divisions run on the vector ALU; everything here is wave-uniform, and saying so keeps what is derived
+        // from it - descriptors, scalar offsets - in scalar registers)
+        tile_m = __builtin_amdgcn_readfirstlane(first_m + tin % gsz);
+        tile_n = __builtin_amdgcn_readfirstlane(tin / gsz);
+        bz = __builtin_amdgcn_readfirstlane(bz);
     };
 
     // ---- compute side: the output tile whose accumulators this workgroup holds ----
@@ -279,6 +290,17 @@ hrn_mfma_kernel(const HrnKArgs a) {
     bool issue_alive = true;
 
     const int lrow = lane / CPR, lpos = lane % CPR;
+    // When the rows that successive load instructions of a wave cover (NW*RPI apart) share their swizzle phase, a
+    // lane's byte offset inside "its" row block is the same for every load and every tile: lane_off.  The row block
+    // itself - tile origin, wave, load index - is a scalar and goes into the buffer descriptor (base advanced by the
+    // block's byte offset, size reduced by it, so that rows past the end of the matrix still read as zeros).  The
+    // issue side then holds two vector registers instead of one per load and spends no vector ALU work per tile.
+    constexpr bool UNI = (SWZ == 0) || ((NW * RPI) % (CPR << (SWZ > 0 ? SWZ - 1 : 0))) == 0;
+    constexpr bool UNI_A = UNI && OP == 0;
+    const uint32_t lane_chunk = (uint32_t)((lpos ^ swz_of_row(wave * RPI + lrow)) * 16);
+    const uint32_t lane_offB = (uint32_t)lrow * (uint32_t)a.ldb * ES + lane_chunk;
+    const uint32_t lane_offA = (uint32_t)lrow * (uint32_t)a.lda * ES + lane_chunk;
+    uint32_t blkA = 0, blkB = 0;                 // byte offset of the wave's first row block of the issue-side tile
     uint32_t voffB[B_LPW];
     // GEMM: byte offset of the lane's chunk in k-tile 0.  Conv: pixel bookkeeping.
     uint32_t voffA[(A_LPW > 0 ? A_LPW : 1)];
@@ -294,14 +316,20 @@ hrn_mfma_kernel(const HrnKArgs a) {
         const int im0 = tile_m * BM, in0 = tile_n * BN;
         baseA = (const char*)a.A + (int64_t)bz * a.sA * ES;
         baseB = (const char*)a.B + (int64_t)bz * a.sB * ES;
+        if constexpr (UNI) {
+            blkB = (uint32_t)(in0 + wave * RPI) * (uint32_t)a.ldb * ES;
+        } else {
 #pragma unroll
-        for (int i = 0; i < B_LPW; ++i) {
-            const int row = (i * NW + wave) * RPI + lrow;
-            const int chunk = lpos ^ swz_of_row(row);
-            const int n = in0 + row;
-            voffB[i] = (n < a.N) ? (uint32_t)n * (uint32_t)a.ldb * ES + chunk * 16 : OOB;
+            for (int i = 0; i < B_LPW; ++i) {
+                const int row = (i * NW + wave) * RPI + lrow;
+                const int chunk = lpos ^ swz_of_row(row);
+                const int n = in0 + row;
+                voffB[i] = (n < a.N) ? (uint32_t)n * (uint32_t)a.ldb * ES + chunk * 16 : OOB;
+            }
         }
-        if constexpr (OP == 0) {
+        if constexpr (UNI_A) {
+            blkA = (uint32_t)(im0 + wave * RPI) * (uint32_t)a.lda * ES;
+        } else if constexpr (OP == 0) {
 #pragma unroll
             for (int i = 0; i < A_LPW; ++i) {
                 const int row = (i * NW + wave) * RPI + lrow;
@@ -350,8 +378,17 @@ hrn_mfma_kernel(const HrnKArgs a) {
     // partly filled one (its chunks past the end of K are masked per lane); the plain form spends no vector ALU work.
     rsrc_t rA_cur, rB_cur;
     uint32_t ks_cur = 0, koff_cur = 0;
+    bool live_cur = false;
+    // descriptor of row block `i` of an operand: base advanced by the block's offset, size reduced by it
+    auto block_rsrc = [&](const char* base, uint32_t bytes, uint32_t blk0, uint32_t ld_bytes, int i) {
+        // (wave-uniform by construction; said explicitly, or the descriptor is treated as a per-lane value)
+        const uint32_t off = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blk0 + (uint32_t)(i * NW * RPI) * ld_bytes));
+        const uint32_t left = (uint32_t)__builtin_amdgcn_readfirstlane((int)((live_cur && bytes > off) ? bytes - off : 0u));
+        return make_rsrc(base + off, left);
+    };
     auto begin_issue = [&]() {
         const bool live = issue_alive && issue_kt < KT;                          // wave-uniform
+        live_cur = live;
         koff_cur = (uint32_t)(kt0 + issue_kt) * BKB;                             // byte offset of the k-tile in a row
         // a dead tile (past the end of K, or past the workgroup's last output tile) reads zeros through empty descriptors
         rB_cur = make_rsrc(baseB, live ? b_bytes : 0u);
@@ -375,7 +412,11 @@ hrn_mfma_kernel(const HrnKArgs a) {
         for (int q = FIRST; q < FIRST + COUNT; ++q) {
             if (q < A_LPW) {
                 const int i = q;
-                if constexpr (OP == 0) {
+                if constexpr (UNI_A) {
+                    uint32_t v = lane_offA;
+                    if constexpr (RAG) { if (koff_rag + lane_chunk >= Kb) v = OOB; }
+                    load_chunk_to_lds(block_rsrc(baseA, a_bytes, blkA, (uint32_t)a.lda * ES, i), sbase + (i * NW + wave) * 1024, v, ks_cur);
+                } else if constexpr (OP == 0) {
                     uint32_t v = voffA[i];
                     if constexpr (RAG) {
                         const int row = (i * NW + wave) * RPI + lrow;
@@ -390,12 +431,18 @@ hrn_mfma_kernel(const HrnKArgs a) {
                 }
             } else {
                 const int i = q - A_LPW;
-                uint32_t v = voffB[i];
-                if constexpr (RAG) {
-                    const int row = (i * NW + wave) * RPI + lrow;
-                    if (koff_rag + (uint32_t)((lpos ^ swz_of_row(row)) * 16) >= Kb) v = OOB;
+                if constexpr (UNI) {
+                    uint32_t v = lane_offB;
+                    if constexpr (RAG) { if (koff_rag + lane_chunk >= Kb) v = OOB; }
+                    load_chunk_to_lds(block_rsrc(baseB, b_bytes, blkB, (uint32_t)a.ldb * ES, i), sbase + A_BYTES + (i * NW + wave) * 1024, v, ks_cur);
+                } else {
+                    uint32_t v = voffB[i];
+                    if constexpr (RAG) {
+                        const int row = (i * NW + wave) * RPI + lrow;
+                        if (koff_rag + (uint32_t)((lpos ^ swz_of_row(row)) * 16) >= Kb) v = OOB;
+                    }
+                    load_chunk_to_lds(rB_cur, sbase + A_BYTES + (i * NW + wave) * 1024, v, ks_cur);
                 }
-                load_chunk_to_lds(rB_cur, sbase + A_BYTES + (i * NW + wave) * 1024, v, ks_cur);
             }
         }
     };
@@ -550,7 +597,12 @@ hrn_mfma_kernel(const HrnKArgs a) {
     // ---- epilogue of the compute-side tile (c_bz, m0, n0) ----
     // MFMA was issued as (B fragment, A fragment), so a lane holds 4 consecutive n for one m:
     //   m = lr, n = (r/4)*8 + lq*4 + r%4   (32x32)     m = lr, n = lq*4 + r   (16x16)
-    auto store_tile = [&]() {
+    auto store_tile = [&]() __attribute__((always_inline)) {
+        // the lane's coordinates, re-derived from values the compiler cannot trace back past this point: otherwise it
+        // computes the epilogue's addresses in front of the k-loop and keeps them in registers all the way through it
+        int lane_e = lane, lr_e, lq_e;
+        asm volatile("" : "+v"(lane_e));
+        lr_e = lane_e % MT; lq_e = lane_e / MT;
         char* const epi = CW ? win : lds + EPI_OFF;
         int* bs_lds = (int*)epi;
         if constexpr (DT == 1) {
@@ -562,12 +614,12 @@ hrn_mfma_kernel(const HrnKArgs a) {
                 int s = bsum[j];
 #pragma unroll
                 for (int d = MT; d < 64; d <<= 1) s += __shfl_xor(s, d, 64);
-                if (lq == 0) bs_lds[wm_idx * BN + wn_idx * WTN + j * MT + lr] = s;
+                if (lq_e == 0) bs_lds[wm_idx * BN + wn_idx * WTN + j * MT + lr_e] = s;
             }
             if constexpr (PERS) wait_and_barrier<63, 0>();
             else __syncthreads();
         }
-        // column sums of the 4 consecutive outputs a lane holds, all wave rows added
+        // column sums of the 4 consecutive outputs a lane_e holds, all wave rows added
         auto colsum4 = [&](int nl) {
             v4i bs = *(const v4i*)(bs_lds + nl);
 #pragma unroll
@@ -576,10 +628,9 @@ hrn_mfma_kernel(const HrnKArgs a) {
         };
 
         char* Cb = (char*)a.C + ((int64_t)slice * a.batch + c_bz) * a.sC * OES;
-        const bool do_store = !(ABL & 16) || a.K == 0x7fffffff;   // the study switch keeps the stores reachable but never takes them
         if constexpr (EPI >= 1) {
             // LDS-staged epilogue: a wave parks one MFMA row-tile (MT rows x SW columns) of its result in a private,
-            // padded LDS strip, then streams it out with 16 bytes per lane, whole row segments per store instruction.
+            // padded LDS strip, then streams it out with 16 bytes per lane_e, whole row segments per store instruction.
             if constexpr (DT == 0 && !PERS) wait_and_barrier<0, 0>();   // (the int8 path has synchronised above) stages are dead now
             [[maybe_unused]] const rsrc_t rsrcC = make_rsrc(Cb, (uint32_t)a.M * (uint32_t)a.ldc * OES);
             char* strip = epi + EPI_BASE + wave * (MT * EPI_PITCH);
@@ -595,8 +646,8 @@ hrn_mfma_kernel(const HrnKArgs a) {
                         const int j = h * TNS + js;
 #pragma unroll
                         for (int g = 0; g < ACC_N / 4; ++g) {
-                            const int cl = js * MT + g * 8 + lq * 4;         // column inside the strip
-                            char* dst = strip + lr * EPI_PITCH + cl * OES;
+                            const int cl = js * MT + g * 8 + lq_e * 4;         // column inside the strip
+                            char* dst = strip + lr_e * EPI_PITCH + cl * OES;
                             if constexpr (DT == 0 && !SPLITK) {
                                 v4h o;
 #pragma unroll
@@ -619,7 +670,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
                     asm volatile("" ::: "memory");     // LDS serves one wave's requests in order: the reads below see the writes
 #pragma unroll
                     for (int it = 0; it < MT * CPRW / 64; ++it) {
-                        const int c = it * 64 + lane;
+                        const int c = it * 64 + lane_e;
                         const int row = c / CPRW, cc2 = c % CPRW;
                         const v4i val = *(const v4i*)(strip + row * EPI_PITCH + cc2 * 16);
                         const int m = m0 + wm_idx * WTM + i * MT + row;
@@ -630,7 +681,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
                             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(unsigned int __attribute__((ext_vector_type(4))), val), rsrcC, (int)off, 0, 0);
                         } else {
                             char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
-                            if (do_store && m < a.M) {
+                            if (m < a.M) {
                                 if (n + EPC <= a.N) *(v4i*)dst = val;
                                 else if (OES == 2 && n + 4 <= a.N) *(long*)dst = ((long)(uint32_t)val.y << 32) | (uint32_t)val.x;
                             }
@@ -642,14 +693,14 @@ hrn_mfma_kernel(const HrnKArgs a) {
         } else {
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                const int m = m0 + wm_idx * WTM + i * MT + lr;
+                const int m = m0 + wm_idx * WTM + i * MT + lr_e;
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
 #pragma unroll
                     for (int g = 0; g < ACC_N / 4; ++g) {
-                        const int nl = wn_idx * WTN + j * MT + g * 8 + lq * 4;
+                        const int nl = wn_idx * WTN + j * MT + g * 8 + lq_e * 4;
                         const int n = n0 + nl;
-                        if (do_store && m < a.M && n < a.N) {
+                        if (m < a.M && n < a.N) {
                             char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
                             if constexpr (DT == 0 && !SPLITK) {
                                 v4h o;
@@ -677,9 +728,9 @@ hrn_mfma_kernel(const HrnKArgs a) {
 
     // ---- prologue: fill all stages, wait for tile 0 ----
 #pragma unroll
-    for (int s = 0; s < (FD ? FD : NS); ++s) issue_tile(s % NS);
-    wait_and_barrier<((FD ? FD : NS) - 1) * LPT, 0>();
-    read_frags(0, 0, 0);
+    for (int s = 0; s < NS; ++s) issue_tile(s);
+    wait_and_barrier<(NS - 1) * LPT, 0>();
+    if constexpr (SCHED != 2) read_frags(0, 0, 0);
 
     int stage = 0;
     // One k-step: the MFMAs of register buffer `cur`, row-tile by row-tile, with the fragment reads of the next step
@@ -688,44 +739,48 @@ hrn_mfma_kernel(const HrnKArgs a) {
     // come first (the next tile's fragment reads may not pass them: both touch LDS), over the first rows of the last
     // step; reads fill the remaining rows but leave the final row free, so that the barrier of the next tile does
     // not wait for a read that was just issued.
-    auto kstep = [&](auto lastc, const bool rag, const int cur, const int rd_stage_off, const int rd_kk, const int kt,
-                     const int step) {
+    auto kstep = [&](auto lastc, auto mayragc, const bool rag, const int cur, const int rd_stage_off, const int rd_kk,
+                     const int kt, const int step) __attribute__((always_inline)) {
         constexpr bool LAST = decltype(lastc)::value;
-        constexpr int NLD = (LAST && !(ABL & 2)) ? LPT : 0;
+        constexpr bool MAYRAG = decltype(mayragc)::value;
+        constexpr int NLD = LAST ? LPT : 0;
         // rows of the last step that carry the tile's loads: HRN_LSPREAD 0 = none (all loads right behind the barrier),
         // 1 = the first quarter of the rows, 2 = half, 3 = all but the last two; spreading the requests smooths the
         // demand on the L2 (every workgroup of an XCD reaches its barrier at about the same time), at the price of a
-        // later arrival of the tile
-        constexpr int LROWS_WANT = LSPREAD == 0 ? 0 : (LSPREAD == 1 ? TM / 4 : (LSPREAD == 2 ? TM / 2 : TM - 2));
-        constexpr int LROWS = NLD == 0 ? 0 : (LROWS_WANT < 0 ? 0 : (LROWS_WANT > TM - 1 ? TM - 1 : (LROWS_WANT == 0 && LSPREAD > 0 && TM >= 2 ? 1 : LROWS_WANT)));
+        // later arrival of the tile.  The reads of the next step follow, the final row stays free (so that the barrier
+        // of the next tile does not wait for a read that was just issued).
+        constexpr int LWANT = LSPREAD == 0 ? 0 : (LSPREAD == 1 ? TM / 4 : (LSPREAD == 2 ? TM / 2 : TM - 2));
+        constexpr int LROWS = NLD == 0 ? 0 : (LWANT < 1 ? ((LSPREAD > 0 && TM >= 2) ? 1 : 0) : (LWANT > TM - 1 ? TM - 1 : LWANT));
+        constexpr int LFIRST = 0;                                                     // first load row
+        constexpr int RFIRST_ROW = LROWS;                                             // first read row
         constexpr int RROWS_ALL = TM - LROWS;                                         // rows left for the reads
         constexpr int RROWS = RROWS_ALL >= 2 ? RROWS_ALL - 1 : RROWS_ALL;             // ... minus the free final row
-        const bool do_reads = !(ABL & 1) || kt == 0;
         // the ragged form differs in the loads only, so the branch (wave-uniform) goes around just these
         auto loads = [&](auto firstc, auto countc) {
-            if (rag) issue_loads(TrueC{}, stage, firstc, countc);
-            else issue_loads(FalseC{}, stage, firstc, countc);
+            if constexpr (MAYRAG) {
+                if (rag) issue_loads(TrueC{}, stage, firstc, countc);
+                else issue_loads(FalseC{}, stage, firstc, countc);
+            } else {
+                issue_loads(FalseC{}, stage, firstc, countc);
+            }
         };
         if constexpr (LROWS == 0 && NLD > 0) loads(std::integral_constant<int, 0>{}, std::integral_constant<int, NLD>{});
         v4i av = a_operand(cur, 0);
         auto row = [&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            if constexpr (i < LROWS) {
-                constexpr int f = NLD * i / LROWS, n = NLD * (i + 1) / LROWS - f;
+            if constexpr (i >= RFIRST_ROW && i - RFIRST_ROW < RROWS) {
+                constexpr int f = NRD * (i - RFIRST_ROW) / RROWS, n = NRD * (i - RFIRST_ROW + 1) / RROWS - f;
+#pragma unroll
+                for (int r = f; r < f + n; ++r) read_slot(cur ^ 1, rd_stage_off, rd_kk, r);
+            }
+            if constexpr (LROWS > 0 && i >= LFIRST && i - LFIRST < LROWS) {
+                constexpr int f = NLD * (i - LFIRST) / LROWS, n = NLD * (i - LFIRST + 1) / LROWS - f;
                 loads(std::integral_constant<int, f>{}, std::integral_constant<int, n>{});
-            } else if constexpr (i - LROWS < RROWS) {
-                constexpr int f = NRD * (i - LROWS) / RROWS, n = NRD * (i - LROWS + 1) / RROWS - f;
-                if (do_reads) {
-#pragma unroll
-                    for (int r = f; r < f + n; ++r) read_slot(cur ^ 1, rd_stage_off, rd_kk, r);
-                }
             }
-            if (!(ABL & 8)) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = mfma(fb[cur][j], av, acc[i][j]);
-            }
+            for (int j = 0; j < TN; ++j) acc[i][j] = mfma(fb[cur][j], av, acc[i][j]);
             if constexpr (i + 1 < TM) av = a_operand(cur, i + 1);      // ready before the next row's MFMAs ask for it
-            if constexpr (SCHED == 1) __builtin_amdgcn_sched_barrier(0);
+            if constexpr (SCHED >= 1) __builtin_amdgcn_sched_barrier(0);
         };
         auto rows = [&](auto self, auto ic) -> void {
             row(ic);
@@ -737,7 +792,9 @@ hrn_mfma_kernel(const HrnKArgs a) {
     };
     // One k-tile.  P = register buffer that holds the fragments of its first k-step (the buffers alternate per
     // k-step, so with an odd number of k-steps per tile P alternates per tile).
-    auto tile_body = [&](auto pc, const int kt, const bool stores_between) {
+    // MAYRAG: the k-tile this iteration fetches may be the partly filled last one of K (only then is the per-lane
+    // masking of the loads compiled in; every other iteration runs the branch-free form).
+    auto tile_body = [&](auto pc, auto mayragc, const int kt, const bool stores_between) __attribute__((always_inline)) {
         constexpr int P = decltype(pc)::value;
         const int stage_off = stage * STAGE_BYTES;
         const int next_stage = (stage + 1 == NS) ? 0 : stage + 1;
@@ -750,36 +807,155 @@ hrn_mfma_kernel(const HrnKArgs a) {
                 if constexpr (PERS) {
                     if (stores_between && kt <= NS - 2) wait_and_barrier<(NS - 2) * LPT + STORES_PER_TILE, 0>();
                     else wait_and_barrier<(NS - 2) * LPT, 0>();
-                } else if constexpr (ABL & 4) {
-                    wait_only<((FD ? FD : NS) - 2) * LPT, 0>();
                 } else {
-                    wait_and_barrier<((FD ? FD : NS) - 2) * LPT, 0>();
+                    wait_and_barrier<(NS - 2) * LPT, 0>();
                 }
                 const bool rag = begin_issue();
                 conv_tap();
                 advance_reader();
-                kstep(TrueC{}, rag, cur, next_stage * STAGE_BYTES, 0, kt, kt * KS + kk);
-                if (!(ABL & 2)) end_issue();
+                kstep(TrueC{}, mayragc, rag, cur, next_stage * STAGE_BYTES, 0, kt, kt * KS + kk);
+                end_issue();
             } else {
-                kstep(FalseC{}, false, cur, stage_off, kk + 1, kt, kt * KS + kk);
+                kstep(FalseC{}, FalseC{}, false, cur, stage_off, kk + 1, kt, kt * KS + kk);
             }
         }
         stage = next_stage;
     };
     using P0 = std::integral_constant<int, 0>;
     using P1 = std::integral_constant<int, 1>;
-    auto run_tile = [&](const bool stores_between) {
+    // Iteration kt fetches k-tile kt + NS of the stream, so only iteration KT - 1 - NS can meet the partly filled last
+    // k-tile (a persistent stream shorter than NS + 1 k-tiles wraps more than once: every iteration may then).
+    const bool k_ragged = (Kb % BKB) != 0;
+    const int kt_rag = k_ragged ? KT - 1 - NS : -1;
+    const bool rag_any = k_ragged && PERS && kt_rag < 0;
+    // the k-tiles [from, to) of the compute-side tile; P0/P1 alternate when a k-tile holds an odd number of k-steps
+    auto tiles = [&](auto mayragc, const int from, const int to, const bool stores_between) __attribute__((always_inline)) {
         if constexpr (KS % 2 == 0) {
-            for (int kt = 0; kt < KT; ++kt) tile_body(P0{}, kt, stores_between);
+            for (int kt = from; kt < to; ++kt) tile_body(P0{}, mayragc, kt, stores_between);
         } else {
-            for (int kt = 0; kt < KT; kt += 2) {
-                tile_body(P0{}, kt, stores_between);
-                if (kt + 1 < KT) tile_body(P1{}, kt + 1, stores_between);
+            int kt = from;
+            if (kt < to && (kt & 1)) { tile_body(P1{}, mayragc, kt, stores_between); ++kt; }
+            for (; kt < to; kt += 2) {
+                tile_body(P0{}, mayragc, kt, stores_between);
+                if (kt + 1 < to) tile_body(P1{}, mayragc, kt + 1, stores_between);
             }
+        }
+    };
+    auto run_tile = [&](const bool stores_between) __attribute__((always_inline)) {
+        if (rag_any) {
+            tiles(TrueC{}, 0, KT, stores_between);
+        } else {
+            // three loops in a row instead of a test inside one: the hot loops carry no ragged-tile code at all
+            const int cut = min(max(kt_rag, 0), KT);
+            tiles(FalseC{}, 0, cut, stores_between);
+            if (kt_rag >= 0) tiles(TrueC{}, cut, min(cut + 1, KT), stores_between);
+            tiles(FalseC{}, kt_rag >= 0 ? min(cut + 1, KT) : cut, KT, stores_between);
         }
         store_tile();
     };
-    if constexpr (PERS) {
+    // ---- SCHED 2: two wave groups half a k-step apart ("ping-pong") ----
+    // Waves w and w + 4 run on the same SIMD.  Group 0 (waves 0-3) and group 1 (waves 4-7) alternate between two kinds
+    // of phase, one barrier apart: a memory phase (read the fragments of one k-step from LDS into the single register
+    // buffer, flip the uint8 sign bits, add up the column sums) and a matrix phase (nothing but that step's MFMAs).
+    // While one wave of a SIMD multiplies, the other waits for LDS and for a slot in the vector-memory queue, so those
+    // waits never hold back an MFMA.  Phase 2s: group 0 multiplies step s, group 1 reads step s; phase 2s+1: group 0
+    // reads step s+1, group 1 multiplies step s.  The stage of k-tile t is free once group 1 has read its last step;
+    // in the phase after that every wave issues its share of the loads of k-tile t + NS, and every wave waits for its
+    // own loads of k-tile t + 1 at the end of the phase in which group 1 reads the last step of k-tile t.
+    // fragment reads of the step whose k-offset inside the stage row is `koff` bytes (a runtime value here: the
+    // k-loop of this schedule is not unrolled over the k-steps of a tile, so that every fragment register has one
+    // definition per iteration and stays where it is)
+    auto pp_mem = [&](const int stage_off, const int koff) __attribute__((always_inline)) {
+        const int gk = g16 ^ koff;
+        const char* pb = lds + stage_off + b_lane + gk;
+        const char* pa = lds + stage_off + a_lane + gk;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[0][j] = *(const v4i*)(pb + j * MT * BKB);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[0][i] = *(const v4i*)(pa + i * MT * BKB);
+    };
+    auto pp_ready = [&](const int step) __attribute__((always_inline)) {      // after the reads have landed
+        if constexpr (DT == 1) {
+            // (as volatile statements, so that the sign flips stay in this phase: plain code may be moved past
+            // the barrier into the matrix phase)
+            const int flip = (int)0x80808080;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                asm volatile("v_xor_b32 %0, %4, %0\n\tv_xor_b32 %1, %4, %1\n\tv_xor_b32 %2, %4, %2\n\tv_xor_b32 %3, %4, %3"
+                             : "+v"(fa[0][i].x), "+v"(fa[0][i].y), "+v"(fa[0][i].z), "+v"(fa[0][i].w) : "s"(flip));
+        }
+        bsum_step(0, step);
+    };
+    auto pp_mfma = [&]() __attribute__((always_inline)) {
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) mfma_inplace(fb[0][j], fa[0][i], acc[i][j]);
+        __builtin_amdgcn_s_setprio(0);
+    };
+    auto pp_fence = [&]() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
+    const bool grp1 = wave >= NW / 2;                     // wave-uniform: the group that runs one phase behind
+    // Both groups run the SAME instruction stream - read step s, barrier, multiply step s, barrier, read step s+1 ... -
+    // and group 1 enters it one barrier later, so the two are always in opposite kinds of phase.  Only the fetches of
+    // the next k-tile and the waits for them sit at group-dependent places of the stream (uniform branches around
+    // nothing but those), because they are tied to the moment at which a stage becomes free for BOTH groups.
+    auto pp_loads = [&]() __attribute__((always_inline)) {
+        const bool rag = begin_issue();
+        conv_tap();
+        if (rag) issue_loads(TrueC{}, stage, std::integral_constant<int, 0>{}, std::integral_constant<int, LPT>{});
+        else issue_loads(FalseC{}, stage, std::integral_constant<int, 0>{}, std::integral_constant<int, LPT>{});
+        end_issue();
+    };
+    auto pp_run = [&]() __attribute__((always_inline)) {
+        if (grp1) wait_and_barrier<63, 15>();            // group 1 enters the stream one phase later
+        pp_fence();
+        pp_mem(0, 0);
+        pp_fence();
+        wait_only<63, 0>();
+        pp_ready(0);
+        pp_fence();
+        if (KS == 1 && grp1) wait_only<(NS - 2) * LPT, 15>();
+        wait_and_barrier<63, 15>();
+        pp_fence();
+        int kk = 0;                                      // k-step inside the k-tile
+        const int steps = KT * KS;
+        for (int step = 0; step < steps; ++step) {
+            const bool last = (kk == KS - 1);
+            const int nkk = last ? 0 : kk + 1;
+            const bool next_last = (nkk == KS - 1);
+            const int next_stage = (stage + 1 == NS) ? 0 : stage + 1;
+            // ---- multiply step `step` (group 0: phase 2*step, group 1: one phase later) ----
+            if (last && grp1) pp_loads();                // the stage of this k-tile is free for both groups now
+            pp_fence();
+            pp_mfma();
+            pp_fence();
+            // before the next k-tile is published every wave's share of it has landed (group 0 waits here ...)
+            if (last && !grp1) wait_only<(NS - 2) * LPT, 15>();
+            wait_and_barrier<63, 15>();
+            pp_fence();
+            // ---- read step `step + 1` ----
+            pp_mem((last ? next_stage : stage) * STAGE_BYTES, nkk * KSB);
+            pp_fence();
+            if (last && !grp1) pp_loads();               // group 0 is one phase ahead: the stage is free only now
+            pp_fence();
+            wait_only<63, 0>();
+            pp_ready(step + 1);
+            pp_fence();
+            if (next_last && grp1) wait_only<(NS - 2) * LPT, 15>();      // (... group 1 here)
+            wait_and_barrier<63, 15>();
+            pp_fence();
+            kk = nkk;
+            if (last) stage = next_stage;
+        }
+        if (!grp1) wait_and_barrier<63, 15>();           // ... and group 0 leaves it one phase earlier
+    };
+    if constexpr (SCHED == 2) {
+        static_assert(SCHED != 2 || (NW == 8 && !CW && !PERS && !SPLITK), "the two-group schedule: 8 waves, plain launch");
+        pp_run();
+        mfma_drain();
+        store_tile();
+    } else if constexpr (PERS) {
         for (int ct = blockIdx.x; ct < total; ct += (int)gridDim.x) {
             tile_coords(ct, c_bz, c_tile_m, c_tile_n);
             m0 = c_tile_m * BM; n0 = c_tile_n * BN;

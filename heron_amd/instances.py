@@ -56,6 +56,12 @@ def variant_descs():
     for t in EPILOGUE_VARIANTS + SINGLE_STEP_VARIANTS:
         out.append(D(F16, GEMM, *t, epi=1))
         out.append(D(U8, GEMM, *t, epi=1))
+    # two-group schedule (sched 2): 8 waves, one and two k-steps per tile, 2..4 stages, both MFMA shapes, im2col conv
+    out.append(D(U8, GEMM, 256, 256, 128, 2, 4, 16, 2, 1, sched=2))
+    out.append(D(F16, GEMM, 256, 256, 128, 4, 2, 16, 2, 1, epi=2, sched=2))
+    out.append(D(U8, GEMM, 128, 128, 64, 2, 4, 16, 4, 3, epi=1, sched=2))
+    out.append(D(F16, GEMM, 128, 256, 64, 2, 4, 32, 3, 2, sched=2))
+    out.append(D(F16, CONV, 128, 64, 128, 4, 2, 16, 2, 1, epi=1, sched=2))
     out.append(D(F16, GEMM, 64, 64, 64, 1, 2, 16, 2, 3))
     out.append(D(U8, GEMM, 128, 128, 64, 4, 1, 16, 3, 3))
     out.append(D(F16, CONV, 256, 64, 128, 8, 1, 16, 2, 1, epi=1))

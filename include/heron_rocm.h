@@ -86,7 +86,10 @@ typedef struct hrn_kernel_desc {
                              pass of the library adds them into C (for small M*N with long K: more workgroups than
                              output tiles).  Not with persistent or conv_window. */
     int32_t sched;        /* issue order of a k-step: 1 = the template's own interleaving of fragment reads, tile loads
-                             and MFMAs is pinned with scheduling fences, 0 = left to the compiler under group hints */
+                             and MFMAs is pinned with scheduling fences, 0 = left to the compiler under group hints,
+                             2 = two-group schedule (8 waves, no conv_window / persistent / split_k): waves 0-3 and
+                             4-7 alternate, one barrier apart, between a phase that only reads fragments and one that
+                             only multiplies, with a single fragment register buffer */
     int32_t load_spread;  /* with sched = 1: how far the wave loads of the next k-tile are spread over the MFMA rows of the
                              step that issues them: 0 = all right behind the barrier, 1 = over a quarter of the rows,
                              2 = half, 3 = all but the last two (smoother demand on the L2, later arrival) */
