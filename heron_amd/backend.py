@@ -52,10 +52,10 @@ class KernelDesc(ctypes.Structure):
                 ("stages", ctypes.c_int32), ("swizzle", ctypes.c_int32), ("epilogue", ctypes.c_int32),
                 ("waves_per_eu", ctypes.c_int32), ("conv_window", ctypes.c_int32), ("persistent", ctypes.c_int32),
                 ("split_k", ctypes.c_int32), ("sched", ctypes.c_int32),
-                ("load_spread", ctypes.c_int32)]
+                ("load_spread", ctypes.c_int32), ("colsum", ctypes.c_int32)]
 
     KEYS = ("dtype", "op", "bm", "bn", "bkb", "wm", "wn", "mfma", "stages", "swizzle", "epilogue", "waves_per_eu",
-            "conv_window", "persistent", "split_k", "sched", "load_spread")
+            "conv_window", "persistent", "split_k", "sched", "load_spread", "colsum")
 
     def as_tuple(self):
         return tuple(int(getattr(self, k)) for k in self.KEYS)
@@ -83,12 +83,14 @@ class Problem(ctypes.Structure):
                 ("cstride", ctypes.c_int32), ("cpad", ctypes.c_int32), ("cdil", ctypes.c_int32),
                 ("group_m", ctypes.c_int32),
                 ("cstride_w", ctypes.c_int32), ("cpad_w", ctypes.c_int32), ("cdil_w", ctypes.c_int32),
-                ("split_k", ctypes.c_int32), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t)]
+                ("split_k", ctypes.c_int32), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+                ("bsum", ctypes.c_void_p)]
 
 
 def make_desc(dtype, op=HRN_OP_GEMM, bm=128, bn=128, bkb=128, wm=2, wn=2, mfma=32, stages=2, swizzle=1,
-              epilogue=0, waves_per_eu=0, conv_window=0, persistent=0, split_k=0, sched=1, load_spread=2):
+              epilogue=0, waves_per_eu=0, conv_window=0, persistent=0, split_k=0, sched=1, load_spread=2, colsum=0):
     d = KernelDesc()
+    d.colsum = colsum
     d.conv_window, d.persistent, d.split_k, d.sched, d.load_spread = conv_window, persistent, split_k, sched, load_spread
     d.dtype, d.op, d.bm, d.bn, d.bkb, d.wm, d.wn = dtype, op, bm, bn, bkb, wm, wn
     d.mfma, d.stages, d.swizzle, d.epilogue, d.waves_per_eu = mfma, stages, swizzle, epilogue, waves_per_eu
@@ -144,6 +146,7 @@ SYMBOLS = {
     "hrn_probe_copy": (_i, [_vp, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_probe_launch": (_i, [_i, _i, ctypes.POINTER(_d), _vp]),
     "hrn_pad_rows": (_i, [_vp, _vp, ctypes.c_size_t, _i, _i, _i, _vp]),
+    "hrn_colsum_s8": (_i, [_vp, _vp, _i, _i, _i, _i, ctypes.c_int64, _vp]),
     "hrn_transpose_pad": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "hrn_probe_read": (_i, [_vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_last_error": (ctypes.c_char_p, []),
@@ -242,6 +245,14 @@ def probe_launch(grid=256, repeat=2000, stream=0):
     return out.value
 
 
+def colsum_s8(b_ptr, out_ptr, batch, n, k, ldb=None, stride_b=None, stream=0):
+    """out[b*n + j] = sum_k B[b][j][k] of an int8 operand (device pointers; out holds batch * n int32): the
+    weight-side preparation of a ``colsum`` instance."""
+    ldb = k if ldb is None else ldb
+    stride_b = n * ldb if stride_b is None else stride_b
+    _check(lib().hrn_colsum_s8(b_ptr, out_ptr, batch, n, k, ldb, stride_b, stream))
+
+
 def pad_rows(src_ptr, dst_ptr, rows, c, cp, elem_bytes, stream=0):
     """Zero-pads rows of c elements to cp elements (device pointers, dst holds rows * cp elements)."""
     _check(lib().hrn_pad_rows(src_ptr, dst_ptr, rows, c, cp, elem_bytes, stream))
@@ -294,6 +305,22 @@ class Module:
         problem.workspace_bytes = ws.numel()
         return problem
 
+    def bind_colsum(self, problem, b_ptr, stream=0):
+        """Colsum instances: when the caller supplied no column sums of B (``problem.bsum``), compute them now into a
+        buffer of this module - fresh on every call, since only the caller knows whether B has changed; callers with
+        fixed weights compute them once (``colsum_s8``) and set ``problem.bsum`` themselves."""
+        if not self.desc.colsum or problem.bsum:
+            return problem
+        need = int(problem.batch) * int(problem.n) * 4
+        buf = getattr(self, "_bs", None)
+        if buf is None or buf.numel() < need:
+            import torch
+            self._bs = buf = torch.empty(max(need, 4096), dtype=torch.uint8, device="cuda")
+        colsum_s8(b_ptr, buf.data_ptr(), int(problem.batch), int(problem.n), int(problem.k), int(problem.ldb),
+                  int(problem.stride_b) if problem.op == HRN_OP_GEMM else 0, stream)
+        problem.bsum = buf.data_ptr()
+        return problem
+
     def _launcher(self, problem):
         L = lib()
         if self.desc.op == HRN_OP_CONV2D:
@@ -304,6 +331,7 @@ class Module:
 
     def launch(self, problem, a_ptr, b_ptr, c_ptr, stream=0):
         self.bind_workspace(problem)
+        self.bind_colsum(problem, b_ptr, stream)
         _check(self._launcher(problem)(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, stream))
 
     def launch_splitk_static(self, problem, a_ptr, b_ptr, c_ptr, stream=0):
@@ -313,18 +341,23 @@ class Module:
     def launch_repeat(self, problem, a_ptr, b_ptr, c_ptr, count, stream=0):
         """``count`` back-to-back launches issued from one host call."""
         self.bind_workspace(problem)
+        self.bind_colsum(problem, b_ptr, stream)
         _check(lib().hrn_launch_repeat(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, count, stream))
 
     def time_cold(self, problem, a_ptr, b_ptr, c_ptr, flush_ptr, flush_bytes, repeat=4, stream=0):
         """Seconds of ``repeat`` single launches, each after the caches were flushed with the caller's buffer."""
         self.bind_workspace(problem)
+        self.bind_colsum(problem, b_ptr, stream)
         costs = (_d * repeat)()
         _check(lib().hrn_time_cold(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, flush_ptr, flush_bytes, repeat,
                                    costs, stream))
         return list(costs)
 
     def time(self, problem, a_ptr, b_ptr, c_ptr, number=3, repeat=4, min_repeat_ms=0.0, stream=0):
+        """time_evaluator-style timing of the kernel.  For a colsum instance without ``problem.bsum`` the column
+        sums of B are computed once before the timed launches (weights are fixed while a kernel is timed)."""
         self.bind_workspace(problem)
+        self.bind_colsum(problem, b_ptr, stream)
         costs = (_d * repeat)()
         _check(lib().hrn_time(self._h, ctypes.byref(problem), a_ptr, b_ptr, c_ptr, number, repeat,
                               float(min_repeat_ms), costs, stream))
@@ -335,6 +368,7 @@ class Module:
             lib().hrn_module_free(self._h)
             self._h = None
         self._ws = None
+        self._bs = None
 
     def __del__(self):
         try:

@@ -146,6 +146,8 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (d->persistent && (d->epilogue < 1 || d->conv_window || d->split_k))
         return fail(HRN_E_BADPARAM, "persistent needs the LDS-staged epilogue and neither conv_window nor split_k");
     if (d->split_k && d->conv_window) return fail(HRN_E_BADPARAM, "split_k uses the im2col load path, not conv_window");
+    if (d->colsum < 0 || d->colsum > 1 || (d->colsum && d->dtype != HRN_DT_U8S8))
+        return fail(HRN_E_BADPARAM, "colsum %d (caller-supplied column sums are an option of the u8s8 instances)", d->colsum);
     if (d->sched == 2 && (d->wm * d->wn != 8 || d->conv_window || d->persistent || d->split_k))
         return fail(HRN_E_BADPARAM, "sched 2 (two wave groups) needs 8 waves and neither conv_window, persistent nor split_k");
     Derived r;
@@ -206,9 +208,9 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
 
 std::string desc_key(const hrn_kernel_desc* d, uint64_t srch) {
     char b[256];
-    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_c%d_r%d_k%d_i%d_l%d_%08x", d->dtype, d->op, d->bm, d->bn,
+    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_c%d_r%d_k%d_i%d_l%d_b%d_%08x", d->dtype, d->op, d->bm, d->bn,
              d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu, d->conv_window,
-             d->persistent, d->split_k, d->sched, d->load_spread, (unsigned)(srch ^ (srch >> 32)));
+             d->persistent, d->split_k, d->sched, d->load_spread, d->colsum, (unsigned)(srch ^ (srch >> 32)));
     return b;
 }
 
@@ -295,6 +297,7 @@ int compile_desc(const hrn_kernel_desc* d, double timeout_s, std::string* out_pa
     def("HRN_SPLITK", d->split_k);
     def("HRN_SCHED", d->sched);
     def("HRN_LSPREAD", d->load_spread);
+    def("HRN_COLSUM", d->colsum);
     {
         std::stringstream es(extra);
         std::string tok;
@@ -381,6 +384,11 @@ int fill_args(const hrn_module* mod, const hrn_problem* p, const void* A, const 
     k->sA = p->stride_a; k->sB = p->stride_b; k->sC = p->stride_c;
     k->batch = p->batch;
     k->split = 1;
+    if (d.colsum) {
+        if (!p->bsum || ((uintptr_t)p->bsum % 16))
+            return fail(HRN_E_BADPARAM, "a colsum instance needs hrn_problem.bsum: batch x n int32 column sums of B (hrn_colsum_s8), 16-byte aligned");
+        k->bsum = p->bsum;
+    }
     if ((int64_t)p->ldb * es % 16 || p->ldb < p->k) return fail(HRN_E_BADPARAM, "ldb %d", p->ldb);
     if (p->ldc % 4 || p->ldc < p->n) return fail(HRN_E_BADPARAM, "ldc %d", p->ldc);
     if (d.epilogue >= 1 && !d.split_k && (((int64_t)p->ldc * oes) % 16 || ((uintptr_t)C % 16) || ((int64_t)p->stride_c * oes) % 16))
@@ -540,6 +548,27 @@ int launch(const hrn_module* mod, const hrn_problem* p, const void* A, const voi
     return run_plan(mod, p, plan, p->workspace, (hipStream_t)stream);
 }
 
+// ---- column sums of an int8 matrix ------------------------------------------------------------
+// out[b][n] = sum_k B[b][n][k]: one wave per row, 16 bytes per lane and step, v_dot4 against ones, wave reduction.
+__global__ void __launch_bounds__(256) colsum_s8_kernel(const signed char* __restrict__ B, int* __restrict__ out, int batch, int N,
+                                                        int K, int ldb, int64_t stride_b) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= (int64_t)batch * N) return;
+    const int b = (int)(row / N), n = (int)(row - (int64_t)b * N);
+    const signed char* src = B + (int64_t)b * stride_b + (int64_t)n * ldb;
+    int s = 0;
+    for (int k = lane * 16; k < K; k += 64 * 16) {          // K is a multiple of 16
+        const rv4i v = *(const rv4i*)(src + k);
+        s = __builtin_amdgcn_sdot4(v.x, 0x01010101, s, false);
+        s = __builtin_amdgcn_sdot4(v.y, 0x01010101, s, false);
+        s = __builtin_amdgcn_sdot4(v.z, 0x01010101, s, false);
+        s = __builtin_amdgcn_sdot4(v.w, 0x01010101, s, false);
+    }
+    for (int d = 1; d < 64; d <<= 1) s += __shfl_xor(s, d, 64);
+    if (lane == 0) out[row] = s;
+}
+
 // ---- roofline probes -----------------------------------------------------------------------
 typedef int pv4i __attribute__((ext_vector_type(4)));
 typedef _Float16 pv8h __attribute__((ext_vector_type(8)));
@@ -690,6 +719,17 @@ __global__ void __launch_bounds__(256) probe_empty_kernel(int* sink) {
 }  // namespace
 
 extern "C" {
+
+int hrn_colsum_s8(const void* B, void* bsum, int batch, int n, int k, int ldb, int64_t stride_b, void* stream) {
+    if (!B || !bsum || batch < 1 || n < 1 || k < 16 || k % 16 || ldb < k || ldb % 16 || ((uintptr_t)B % 16) || stride_b % 16)
+        return fail(HRN_E_BADPARAM, "colsum_s8: batch %d, n %d, k %d, ldb %d (k and ldb multiples of 16, B 16-byte aligned)", batch, n, k, ldb);
+    const int64_t rows = (int64_t)batch * n;
+    if ((rows + 3) / 4 >= (1ll << 31)) return fail(HRN_E_BADPARAM, "colsum_s8: too many rows");
+    colsum_s8_kernel<<<(unsigned)((rows + 3) / 4), 256, 0, (hipStream_t)stream>>>((const signed char*)B, (int*)bsum, batch, n, k, ldb, stride_b);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HRN_E_LAUNCH, "colsum_s8: %s", hipGetErrorString(e));
+    return HRN_OK;
+}
 
 int hrn_pad_rows(const void* src, void* dst, size_t rows, int c, int cp, int elem_bytes, void* stream) {
     if (!src || !dst || c < 1 || cp < c || (elem_bytes != 1 && elem_bytes != 2) || (cp * elem_bytes) % 16 || rows > ((size_t)1 << 40))

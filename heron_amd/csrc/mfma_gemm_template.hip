@@ -83,6 +83,13 @@ constexpr bool PERS = (HRN_PERSIST != 0);
 #define HRN_SPLITK 0
 #endif
 constexpr bool SPLITK = (HRN_SPLITK != 0);
+// uint8 path: 1 = the column sums of B (sum_k B[n,k], what the (u8 - 128) x s8 product is short of, times 128) come
+// from the caller (HrnKArgs.bsum: one int32 per column and batch entry, a property of the weights alone) instead of
+// being added up in the k-loop from the B fragments.
+#ifndef HRN_COLSUM
+#define HRN_COLSUM 0
+#endif
+constexpr bool COLSUM = (HRN_DTYPE == 1) && (HRN_COLSUM != 0);
 // Issue order of a k-step: 1 = the source order of the row groups is pinned (a scheduling fence after every row of
 // MFMAs), 0 = the compiler interleaves on its own, guided by group hints (one LDS read per few MFMAs), 2 = the two
 // wave groups of an 8-wave workgroup alternate between a memory phase and a matrix phase (see "SCHED 2" below).
@@ -579,7 +586,7 @@ hrn_mfma_kernel(const HrnKArgs a) {
     // uint8 path: sum_k B[n,k] of the step's B fragments.  The WM waves of one column hold the same fragments, so
     // they take turns: wave row w sums the steps with step % WM == w, the epilogue adds the WM partial sums.
     auto bsum_step = [&](int buf, int step) {
-        if constexpr (DT == 1) {
+        if constexpr (DT == 1 && !COLSUM) {
             if (WM == 1 || (step & (WM - 1)) == wm_idx) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
@@ -609,12 +616,23 @@ hrn_mfma_kernel(const HrnKArgs a) {
             // 128 * sum_k B[n,k] completes the u8 x s8 product computed as (u8-128) x s8
             if constexpr (PERS) wait_and_barrier<63, 0>();     // the stages stay live: LDS traffic only, no drain
             else wait_and_barrier<0, 0>();
+            if constexpr (COLSUM) {
+                // the caller's sums of this tile's BN columns, 16 bytes per lane (N is a multiple of 4); a split-K
+                // slice other than the first adds nothing (the sums cover all of K)
+                for (int q = tid; q < BN / 4; q += NT) {
+                    const int n = n0 + q * 4;
+                    v4i v = {0, 0, 0, 0};
+                    if (slice == 0 && n + 4 <= a.N) v = *(const v4i*)((const int*)a.bsum + (int64_t)c_bz * a.N + n);
+                    *(v4i*)(bs_lds + q * 4) = v;
+                }
+            } else {
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                int s = bsum[j];
+                for (int j = 0; j < TN; ++j) {
+                    int s = bsum[j];
 #pragma unroll
-                for (int d = MT; d < 64; d <<= 1) s += __shfl_xor(s, d, 64);
-                if (lq_e == 0) bs_lds[wm_idx * BN + wn_idx * WTN + j * MT + lr_e] = s;
+                    for (int d = MT; d < 64; d <<= 1) s += __shfl_xor(s, d, 64);
+                    if (lq_e == 0) bs_lds[wm_idx * BN + wn_idx * WTN + j * MT + lr_e] = s;
+                }
             }
             if constexpr (PERS) wait_and_barrier<63, 0>();
             else __syncthreads();
@@ -622,8 +640,10 @@ hrn_mfma_kernel(const HrnKArgs a) {
         // column sums of the 4 consecutive outputs a lane_e holds, all wave rows added
         auto colsum4 = [&](int nl) {
             v4i bs = *(const v4i*)(bs_lds + nl);
+            if constexpr (!COLSUM) {
 #pragma unroll
-            for (int w = 1; w < WM; ++w) bs += *(const v4i*)(bs_lds + w * BN + nl);
+                for (int w = 1; w < WM; ++w) bs += *(const v4i*)(bs_lds + w * BN + nl);
+            }
             return bs;
         };
 

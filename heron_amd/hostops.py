@@ -16,9 +16,23 @@ def _chk(t, dtype):
         raise ValueError("expected a contiguous CUDA tensor of %s, got %s %s" % (dtype, t.dtype, t.device))
 
 
-def gemm(mod, A, Bm, out=None, group_m=8, split_k=0):
+def column_sums(Bm):
+    """Column sums of an int8 operand (N,K) / (b,N,K) / KRSC filter (CO,KH,KW,CI): int32 (N,) / (b,N) / (CO,).  What a
+    ``colsum`` instance takes with the weights; with fixed weights it is computed once."""
+    _chk(Bm, torch.int8)
+    if Bm.dim() == 4:
+        n, k, batch = Bm.shape[0], Bm.shape[1] * Bm.shape[2] * Bm.shape[3], 1
+    else:
+        n, k, batch = Bm.shape[-2], Bm.shape[-1], (Bm.shape[0] if Bm.dim() == 3 else 1)
+    out = torch.empty((batch, n) if Bm.dim() == 3 else (n,), dtype=torch.int32, device=Bm.device)
+    B.colsum_s8(Bm.data_ptr(), out.data_ptr(), batch, n, k, stream=_stream())
+    return out
+
+
+def gemm(mod, A, Bm, out=None, group_m=8, split_k=0, bsum=None):
     """C = A @ Bm.T for A (M,K), Bm (N,K), or batched (b,M,K) x (b,N,K) -> (b,M,N).  ``split_k`` is the number of
-    K slices for a split-K instance (the module supplies the workspace)."""
+    K slices for a split-K instance (the module supplies the workspace).  ``bsum``: the column sums of Bm
+    (``column_sums``) for a ``colsum`` instance; computed on the spot when absent."""
     f16 = mod.desc.dtype == B.HRN_DT_F16
     _chk(A, torch.float16 if f16 else torch.uint8)
     _chk(Bm, torch.float16 if f16 else torch.int8)
@@ -31,6 +45,11 @@ def gemm(mod, A, Bm, out=None, group_m=8, split_k=0):
     if out is None:
         out = torch.empty(oshape, dtype=torch.float16 if f16 else torch.int32, device=A.device)
     p = B.gemm_problem(batch, M, N, K, group_m, split_k)
+    if bsum is not None and mod.desc.colsum:
+        _chk(bsum, torch.int32)
+        if bsum.numel() != batch * N:
+            raise ValueError("bsum holds %d sums, B has %d columns" % (bsum.numel(), batch * N))
+        p.bsum = bsum.data_ptr()
     mod.launch(p, A.data_ptr(), Bm.data_ptr(), out.data_ptr(), _stream())
     return out
 
@@ -44,7 +63,7 @@ def unpack_filter_blocked(Wb):
     return Wb.permute(0, 4, 1, 2, 3, 5).reshape(OC * cb, KH, KW, ICC * 4).contiguous()
 
 
-def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8, split_k=0):
+def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8, split_k=0, bsum=None):
     """X (N,H,W,CI), Wt KRSC (CO,KH,KW,CI) -> (N,HO,WO,CO): fp16 -> fp16, or uint8 x int8 -> int32."""
     f16 = mod.desc.dtype == B.HRN_DT_F16
     _chk(X, torch.float16 if f16 else torch.uint8)
@@ -59,6 +78,11 @@ def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8, split_k
     wo = (W - ((KW - 1) * dw + 1) + 2 * pw) // sw + 1
     if out is None:
         out = torch.empty((N, ho, wo, CO), dtype=torch.float16 if f16 else torch.int32, device=X.device)
+    if bsum is not None and mod.desc.colsum:
+        _chk(bsum, torch.int32)
+        if bsum.numel() != CO:
+            raise ValueError("bsum holds %d sums, the filter has %d output channels" % (bsum.numel(), CO))
+        p.bsum = bsum.data_ptr()
     mod.launch(p, X.data_ptr(), Wt.data_ptr(), out.data_ptr(), _stream())
     return out
 

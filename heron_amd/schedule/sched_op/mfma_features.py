@@ -11,7 +11,7 @@ costs.  Before anything has been measured the estimate itself ranks the candidat
 import math
 
 KNOBS = ('mfma', 'wave_m', 'wave_n', 'tile_m', 'tile_n', 'block_k_bytes', 'conv_window', 'persistent', 'lds_stages',
-         'lds_swizzle', 'waves_per_eu', 'epilogue', 'split_k', 'raster_group_m', 'issue_order', 'load_spread')
+         'lds_swizzle', 'waves_per_eu', 'epilogue', 'split_k', 'raster_group_m', 'issue_order', 'load_spread', 'column_sums')
 DERIVED = ('block_m', 'block_n', 'waves', 'k_steps', 'k_tiles', 'grid_m', 'grid_n', 'lds_bytes', 'window_bytes',
            'regs_per_lane', 'loads_per_tile')
 

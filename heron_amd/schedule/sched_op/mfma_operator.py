@@ -32,7 +32,7 @@ class TemplateSchedule:
         return B.make_desc(dtype, op, p['bm'], p['bn'], p['bkb'], p['wm'], p['wn'], p['mfma'], p['stages'],
                            p['swizzle'], p.get('epilogue', 0), p['waves_per_eu'],
                            p.get('conv_window', 0), p.get('persistent', 0), 1 if p.get('split_k', 1) > 1 else 0,
-                           p.get('sched', 1), p.get('load_spread', 2))
+                           p.get('sched', 1), p.get('load_spread', 2), p.get('colsum', 0))
 
     def to_problem(self):
         from ... import backend as B
@@ -507,9 +507,13 @@ class rasterOp(schedOp):
         gm = self.knob(ctx, stage_name, 'raster_group_m', [1, 2, 4, 8, 16, 32], 8)
         sc = self.knob(ctx, stage_name, 'issue_order', [0, 1], 1)
         sp = self.knob(ctx, stage_name, 'load_spread', [0, 1, 2, 3], 2)
+        # uint8 x int8: where the column sums of B come from (0 = added up in the kernel's k-loop, 1 = supplied with
+        # the weights, hrn_colsum_s8); fp16 has no such term
+        cs = self.knob(ctx, stage_name, 'column_sums', [0, 1] if s.info['kind'] == 'u8s8' else [0], 0)
         s.params['group_m'] = km.get_val(gm)
         s.params['sched'] = km.get_val(sc)
         s.params['load_spread'] = km.get_val(sp)
+        s.params['colsum'] = km.get_val(cs)
         ctx.addSchedDesc("raster group_m = %s, issue order = %s\n" % (s.params['group_m'], s.params['sched']))
 
 

@@ -93,6 +93,9 @@ typedef struct hrn_kernel_desc {
     int32_t load_spread;  /* with sched = 1: how far the wave loads of the next k-tile are spread over the MFMA rows of the
                              step that issues them: 0 = all right behind the barrier, 1 = over a quarter of the rows,
                              2 = half, 3 = all but the last two (smoother demand on the L2, later arrival) */
+    int32_t colsum;       /* u8s8 only: the kernel computes (u8 - 128) x s8 on the signed MFMA and adds 128 * sum_k B[n,k];
+                             0 = it adds those column sums up itself from the B fragments in its k-loop, 1 = it takes
+                             them from hrn_problem.bsum (they depend on the weights alone: hrn_colsum_s8 makes them) */
 } hrn_kernel_desc;
 
 /* Resource usage of a built instance, for cross-checks of the constraint set. */
@@ -132,6 +135,9 @@ typedef struct hrn_problem {
     int32_t split_k;
     void* workspace;
     size_t workspace_bytes;
+    /* colsum instances only (hrn_kernel_desc.colsum = 1): device pointer to batch x n int32 column sums of B,
+     * bsum[b*n + j] = sum_k B[b][j][k] (conv: over the whole filter of output channel j), 16-byte aligned */
+    const void* bsum;
 } hrn_problem;
 
 typedef struct hrn_module hrn_module;
@@ -219,6 +225,15 @@ int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const v
  */
 int hrn_time_cold(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C,
                   void* flush_buf, size_t flush_bytes, int repeat, double* costs_out, void* stream);
+
+/*
+ * Column sums of an int8 operand: bsum[b*n + j] = sum_k B[b][j][k] for B (batch, n, k) with leading dimension ldb and
+ * batch stride stride_b (elements = bytes); k and ldb multiples of 16.  This is the weight-side preparation of the
+ * colsum instances, the counterpart of the reference's pre-packed weight operand: ops/x86/dense.py:7-9 takes the
+ * weights already blocked as (N/16, K/4, 16, 4), so what depends on the weights alone is done once, outside the
+ * operator.  Both buffers are caller-owned device memory; bsum holds batch * n int32.
+ */
+int hrn_colsum_s8(const void* B, void* bsum, int batch, int n, int k, int ldb, int64_t stride_b, void* stream);
 
 /*
  * Channel padding pre-stage: copies `rows` rows of `c` elements (1 or 2 bytes each) from `src` to rows of `cp`

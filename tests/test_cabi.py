@@ -35,7 +35,7 @@ def header_struct(name):
         decl = decl.strip()
         if not decl:
             continue
-        ctype, names = re.match(r"((?:u?int\d+_t|size_t|char|void\s*\*))\s*(.*)", decl, flags=re.S).groups()
+        ctype, names = re.match(r"((?:u?int\d+_t|size_t|char|(?:const\s+)?void\s*\*))\s*(.*)", decl, flags=re.S).groups()
         for n in names.split(","):
             m = re.match(r"\s*(\w+)(?:\[(\d+)\])?\s*$", n)
             out.append((m.group(1), ctype.replace(" ", ""), int(m.group(2) or 0)))
@@ -43,7 +43,7 @@ def header_struct(name):
 
 
 C_TYPES = {"int32_t": ctypes.c_int32, "int64_t": ctypes.c_int64, "uint64_t": ctypes.c_uint64, "size_t": ctypes.c_size_t,
-           "void*": ctypes.c_void_p, "char": ctypes.c_char}
+           "void*": ctypes.c_void_p, "constvoid*": ctypes.c_void_p, "char": ctypes.c_char}
 
 
 def test_struct_layouts_match_header():
@@ -55,7 +55,7 @@ def test_struct_layouts_match_header():
         assert [n for n, _ in have] == [n for n, _ in want], name
         for (n, th), (_, tw) in zip(have, want):
             assert ctypes.sizeof(th) == ctypes.sizeof(tw) and th._type_ == tw._type_, (name, n)
-    assert ctypes.sizeof(B.KernelDesc) == 17 * 4
+    assert ctypes.sizeof(B.KernelDesc) == 18 * 4
     assert B.KernelDesc.KEYS == tuple(n for n, _ in B.KernelDesc._fields_)
 
 

@@ -191,6 +191,42 @@ INT8_CONV_CASES = [
 ]
 
 
+def test_caller_supplied_column_sums(hrn):
+    """colsum instances: hrn_colsum_s8 equals the sum over K (int64 numpy); the product with the sums handed over
+    explicitly, with the sums made on the spot, and of the in-kernel instance are all the oracle's, bit for bit -
+    GEMM, batched, ragged; a launch through the C ABI without the sums is refused, not mis-computed."""
+    import ctypes
+    rng = np.random.default_rng(21)
+    Bm = rng.integers(-128, 128, (3, 200, 272), dtype=np.int8)
+    Bm[0, 0, :] = -128
+    Bm[1, 5, :] = 127
+    got = hostops.column_sums(dev(Bm)).cpu().numpy()
+    assert got.dtype == np.int32 and np.array_equal(got, Bm.astype(np.int64).sum(axis=2))
+    Wt = rng.integers(-128, 128, (48, 3, 3, 32), dtype=np.int8)
+    assert np.array_equal(hostops.column_sums(dev(Wt)).cpu().numpy(), Wt.astype(np.int64).sum(axis=(1, 2, 3)))
+    m = mod_for(instances.D(instances.U8, instances.GEMM, 64, 128, 256, 1, 2, 16, 2, 1, epi=1, colsum=1))
+    for i, (M, K, N) in enumerate([(64, 64, 64), (300, 1040, 520), (100, 208, 72)]):
+        A, B2 = workloads.gemm_u8s8_inputs(M, K, N, seed=400 + i)
+        ref = oracle.gemm_int64_numpy(A, B2).astype(np.int32)
+        dB = dev(B2)
+        assert np.array_equal(hostops.gemm(m, dev(A), dB, bsum=hostops.column_sums(dB)).cpu().numpy(), ref)
+        assert np.array_equal(hostops.gemm(m, dev(A), dB).cpu().numpy(), ref)
+    A = rng.integers(0, 256, (3, 96, 272), dtype=np.uint8)
+    assert np.array_equal(hostops.gemm(m, dev(A), dev(Bm)).cpu().numpy(), oracle.bmm_u8s8s32_scalar(A, Bm))
+    # extremes: 255 x -128 over all of K with the sums supplied
+    A = np.full((64, 8192), 255, np.uint8)
+    B3 = np.full((64, 8192), -128, np.int8)
+    assert int(hostops.gemm(m, dev(A), dev(B3)).cpu().numpy()[0, 0]) == -267386880
+    # the raw entry point refuses a colsum instance without the sums
+    A, B2 = workloads.gemm_u8s8_inputs(64, 64, 64, seed=1)
+    dA, dB, out = dev(A), dev(B2), torch.empty((64, 64), dtype=torch.int32, device="cuda")
+    p = B.gemm_problem(1, 64, 64, 64)
+    rc = B.lib().hrn_launch_gemm_u8s8(m._h, ctypes.byref(p), dA.data_ptr(), dB.data_ptr(), out.data_ptr(), 0)
+    assert rc == B.HRN_E_BADPARAM and b"bsum" in B.lib().hrn_last_error()
+    # and fp16 instances have no such option
+    assert not B.check_desc(instances.D(instances.F16, instances.GEMM, 128, 128, 128, 2, 2, 32, 2, 1, colsum=1))
+
+
 @pytest.mark.parametrize("desc", instances.int8_conv_descs(), ids=lambda d: "-".join(map(str, d.as_tuple())))
 def test_conv2d_nhwc_u8s8_bit_exact(desc, hrn):
     m = mod_for(desc)

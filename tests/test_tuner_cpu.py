@@ -96,7 +96,7 @@ def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
     t = Task("t", getOpFromName(op), shape + [dtype, dtype], "rocm")
     t.config = cfg
     t.make_stage_schedules()
-    assert len(t.knob_manager.knob_names) == 16 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
+    assert len(t.knob_manager.knob_names) == 17 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
     seen = set()
     for _ in range(40):
         km = copy.deepcopy(t.knob_manager)
