@@ -12,7 +12,14 @@ then until two consecutive 20-launch groups agree within 2 %); this does not dep
 launches, then exactly --steps launches bracketed by torch.cuda.synchronize() for ``value`` / ``ms_per_step`` and by
 HIP events on the launch stream for ``config.kernel_ms`` (what ``roofline.achieved`` is computed from).  Rows bounded by
 HBM are also timed cold - every launch after 1 GiB was streamed through the caches - and their roofline fraction
-is the cold one: back-to-back launches of a 126 MB problem run out of the 256 MB memory-side cache.
+is the cold one: back-to-back launches of a 126 MB problem run out of the 256 MB memory-side cache.  Next to it stands
+the like-for-like floor of such a launch: a kernel that only reads the workload's input bytes and writes its output
+bytes, one launch after the same flush (``floor_us_cold``, ``frac_of_floor``).
+
+A uint8 instance may take the column sums of B with the weights (``colsum`` instances): they depend on the weights
+alone, as the reference's pre-packed weight operand does, and are made once, outside the timed region; the line says
+so (``config.weights``) and also gives the figure with that pass counted into every step (``with_colsum_pass``).
+``stable`` repeats the three GEMM figures under fixed names, whichever workload is the headline.
 
 ``cpu_baseline`` times the CPU oracle's DL Boost-style GEMM (AVX512-VNNI 16x4 micro-kernel, all host cores) on the
 same 8192^3 problem and checks the first rows of the very buffer that was timed against it.
@@ -120,11 +127,27 @@ def measure(torch, B, w, steps, warmup, keep_rows=0, cold=False):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
     out = {"wall_s": wall, "kernel_s": e0.elapsed_time(e1) * 1e-3 / steps, "settle_ms": spent, "info": dict(mod.info)}
+    if inst.desc.colsum:
+        # the column sums of B were made once (first launch above); what that pass costs when it is counted in
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(20):
+            B.colsum_s8(pb, int(prob.bsum), int(prob.batch), int(prob.n), int(prob.k), int(prob.ldb),
+                        int(prob.stride_b) if prob.op == B.HRN_OP_GEMM else 0, stream)
+        e1.record()
+        e1.synchronize()
+        out["colsum_pass_s"] = e0.elapsed_time(e1) * 1e-3 / 20
     if cold:
         flush = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
         costs = mod.time_cold(prob, pa, pb, pc, flush.data_ptr(), flush.numel(), repeat=9, stream=stream)
         out["cold_s"] = sorted(costs)[len(costs) // 2]
-        del flush
+        # the floor of that launch: nothing but the algorithmic traffic, same flush, one dispatch
+        rd = (a.numel() * a.element_size() + b.numel() * b.element_size() + 15) // 16 * 16
+        wr = (c.numel() * c.element_size() + 15) // 16 * 16
+        src = torch.empty(rd, dtype=torch.uint8, device="cuda")
+        floor = B.probe_traffic_cold(src.data_ptr(), rd, pc, wr, flush.data_ptr(), flush.numel(), repeat=9, stream=stream)
+        out["floor_s"] = sorted(floor)[len(floor) // 2] * 1e-6
+        del flush, src
     if keep_rows:
         out["rows"] = c.reshape(-1, c.shape[-1])[:keep_rows].cpu().numpy()
     mod.close()
@@ -306,6 +329,15 @@ def main():
     }
     if "cold_s" in r:
         line["config"]["kernel_ms_cold"] = r["cold_s"] * 1e3
+        line["config"]["floor_us_cold"] = r["floor_s"] * 1e6
+        line["roofline"]["frac_of_floor"] = r["floor_s"] / r["cold_s"]
+    if "colsum_pass_s" in r:
+        line["config"]["weights"] = ("column sums of B prepared once with the weights (hrn_colsum_s8), outside the timed "
+                                     "region, like the reference's pre-packed weight operand (ops/x86/dense.py:7-9)")
+        line["config"]["colsum_pass_ms"] = r["colsum_pass_s"] * 1e3
+        line["with_colsum_pass"] = {"ms_per_step": (r["wall_s"] + r["colsum_pass_s"]) * 1e3,
+                                    "value": w["ops"] / (r["wall_s"] + r["colsum_pass_s"]) / 1e12}
+    stable = {args.workload: w["ops"] / r["wall_s"] / 1e12}
     if not args.only:
         line["peaks"] = {"published": {"mfma_f16_TFLOPs": workloads.PEAK_FP16_TFLOPS, "mfma_i8_TOPs": workloads.PEAK_INT8_TOPS,
                                        "hbm_GBs": workloads.PEAK_HBM_GBS}, "used": "published"}
@@ -333,13 +365,22 @@ def main():
                    "frac_of_mfma_peak": ww["ops"] / rr["kernel_s"] / 1e12 / peak, "roofline": rf}
             if "cold_s" in rr:
                 row["kernel_ms_cold"] = rr["cold_s"] * 1e3
+                row["floor_us_cold"] = rr["floor_s"] * 1e6
+                rf["frac_of_floor"] = rr["floor_s"] / rr["cold_s"]
                 row["roofline_timed"] = "cold: every launch after 1 GiB was streamed through the caches"
+            if "colsum_pass_s" in rr:
+                row["colsum_pass_ms"] = rr["colsum_pass_s"] * 1e3
+            stable[name] = row["value"]
             also.append(row)
         line["also"] = also
         try:
             line["cpu_baseline"] = cpu_baseline(workloads, r.get("rows") if args.workload == HEADLINE else None)
         except Exception as e:  # noqa: BLE001 - the GPU figures above are still worth printing
             line["cpu_baseline"] = {"value": None, "unit": None, "cores": 0, "kind": "port", "sample": "failed: %r" % (e,)}
+    # fixed names for the three GEMM figures, whichever of them is the headline (the headline was the fp16 4096^3
+    # GEMM in the first revision of this file and is the u8s8 8192^3 GEMM since)
+    line["stable"] = {"gemm_f16_4096_TFLOPs": stable.get("gemm_f16_4096"), "gemm_f16_8192_TFLOPs": stable.get("gemm_f16_8192"),
+                      "gemm_u8s8_8192_TOPs": stable.get("gemm_u8s8_8192")}
     print(json.dumps(line))
 
 

@@ -149,6 +149,7 @@ SYMBOLS = {
     "hrn_colsum_s8": (_i, [_vp, _vp, _i, _i, _i, _i, ctypes.c_int64, _vp]),
     "hrn_transpose_pad": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "hrn_probe_read": (_i, [_vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
+    "hrn_probe_traffic_cold": (_i, [_vp, ctypes.c_size_t, _vp, ctypes.c_size_t, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_last_error": (ctypes.c_char_p, []),
     "hrn_version": (ctypes.c_char_p, []),
 }
@@ -268,6 +269,14 @@ def probe_read(src_ptr, nbytes, repeat=10, stream=0):
     out = ctypes.c_double()
     _check(lib().hrn_probe_read(src_ptr, nbytes, repeat, ctypes.byref(out), stream))
     return out.value
+
+
+def probe_traffic_cold(src_ptr, read_bytes, dst_ptr, write_bytes, flush_ptr, flush_bytes, repeat=5, stream=0):
+    """Microseconds of ``repeat`` single cold launches of a kernel that only reads ``read_bytes`` and writes
+    ``write_bytes``: the floor of a workload's cold launch (same flush as ``Module.time_cold``)."""
+    out = (_d * repeat)()
+    _check(lib().hrn_probe_traffic_cold(src_ptr, read_bytes, dst_ptr, write_bytes, flush_ptr, flush_bytes, repeat, out, stream))
+    return list(out)
 
 
 def probe_copy(src_ptr, dst_ptr, nbytes, repeat=10, stream=0):

@@ -522,10 +522,14 @@ static __device__ __align__(256) unsigned char scratch[HRN_STATIC_WORKSPACE_BYTE
 constexpr int kMaxDevices = 64;
 void* g_scratch_ptr[kMaxDevices];
 bool g_scratch_known[kMaxDevices];
+hipEvent_t g_scratch_done[kMaxDevices];      // recorded behind the last launch that used the device's workspace ...
+hipStream_t g_scratch_stream[kMaxDevices];   // ... on this stream
+bool g_scratch_used[kMaxDevices];
 std::mutex g_scratch_mutex;
 
-// address of `scratch` on the current device (looked up on the first call per device)
-int static_scratch(void** out) {
+// Address of `scratch` on the current device and the event that orders its users: set up on the first call per
+// device (hrn_build does it for split-K instances, so that a launch - possibly under graph capture - finds it done).
+int static_scratch(void** out, int* dev_out = nullptr) {
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices) return fail(HRN_E_BADPARAM, "device index %d", dev);
@@ -534,10 +538,12 @@ int static_scratch(void** out) {
         void* ptr = nullptr;
         HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
         if (!ptr) return fail(HRN_E_LAUNCH, "hipGetSymbolAddress returned a null address");
+        HIP_TRY(hipEventCreateWithFlags(&g_scratch_done[dev], hipEventDisableTiming));
         g_scratch_ptr[dev] = ptr;
         g_scratch_known[dev] = true;
     }
     *out = g_scratch_ptr[dev];
+    if (dev_out) *dev_out = dev;
     return HRN_OK;
 }
 
@@ -711,6 +717,24 @@ __global__ void __launch_bounds__(256) probe_read_kernel(const pv4i* __restrict_
     asm volatile("" ::"v"(keep));   // keeps the loads live; nothing is stored
 }
 
+// reads `r16` 16-byte words and writes `w16` of them (the words it read, as far as they go): the plainest kernel that
+// moves a workload's algorithmic bytes
+__global__ void __launch_bounds__(256) probe_traffic_kernel(const pv4i* __restrict__ src, size_t r16, pv4i* __restrict__ dst, size_t w16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t n = r16 > w16 ? r16 : w16;
+    pv4i acc = {0, 0, 0, 0};
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += 2 * stride) {
+        const size_t j = i + stride;
+        pv4i v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+        if (i < r16) v0 = src[i];
+        if (j < r16) v1 = src[j];
+        if (i < w16) dst[i] = v0; else acc |= v0;
+        if (j < w16) dst[j] = v1; else acc |= v1;
+    }
+    const int keep = acc.x | acc.y | acc.z | acc.w;
+    asm volatile("" ::"v"(keep));
+}
+
 // does nothing: what the device needs to start and retire one dispatch of `grid` workgroups
 __global__ void __launch_bounds__(256) probe_empty_kernel(int* sink) {
     if (sink && threadIdx.x == 0x7fffffff) *sink = 0;
@@ -780,6 +804,34 @@ int hrn_probe_read(const void* src, size_t bytes, int repeat, double* gbs_out, v
     (void)hipEventElapsedTime(&ms, e0, e1);
     if (e != hipSuccess) return fail(HRN_E_LAUNCH, "probe: %s", hipGetErrorString(e));
     *gbs_out = (double)bytes * repeat / (ms * 1e-3) / 1e9;
+    return HRN_OK;
+}
+
+int hrn_probe_traffic_cold(const void* src, size_t read_bytes, void* dst, size_t write_bytes, void* flush_buf,
+                           size_t flush_bytes, int repeat, double* us_out, void* stream) {
+    if (!src || !dst || !us_out || !flush_buf || read_bytes % 16 || write_bytes % 16 || (read_bytes == 0 && write_bytes == 0) ||
+        repeat < 1 || flush_bytes < (64u << 20))
+        return fail(HRN_E_BADPARAM, "probe arguments (16-byte multiples, flush buffer >= 64 MiB)");
+    int dev = 0;
+    hipDeviceProp_t pr;
+    HIP_TRY(hipGetDevice(&dev));
+    HIP_TRY(hipGetDeviceProperties(&pr, dev));
+    hipStream_t st = (hipStream_t)stream;
+    EventPair ev;
+    HIP_TRY(ev.create());
+    const size_t half16 = flush_bytes / 32;
+    const int grid = pr.multiProcessorCount * 8;
+    for (int r = 0; r < repeat; ++r) {
+        // the same flush as hrn_time_cold: one half of the buffer streamed into the other
+        probe_copy_kernel<<<pr.multiProcessorCount * 16, 256, 0, st>>>((const pv4i*)flush_buf, (pv4i*)flush_buf + half16, half16);
+        (void)hipEventRecord(ev.e0, st);
+        probe_traffic_kernel<<<grid, 256, 0, st>>>((const pv4i*)src, read_bytes / 16, (pv4i*)dst, write_bytes / 16);
+        (void)hipEventRecord(ev.e1, st);
+        if (hipEventSynchronize(ev.e1) != hipSuccess) return fail(HRN_E_LAUNCH, "probe: %s", hipGetErrorString(hipGetLastError()));
+        float ms = 0;
+        (void)hipEventElapsedTime(&ms, ev.e0, ev.e1);
+        us_out[r] = (double)ms * 1e3;
+    }
     return HRN_OK;
 }
 
@@ -934,6 +986,12 @@ int hrn_build(const hrn_kernel_desc* desc, double timeout_s, hrn_module** out) {
         delete m;
         return fail(HRN_E_LOAD, "hipModuleGetFunction: %s", hipGetErrorString(e));
     }
+    if (desc->split_k) {
+        // hrn_launch_splitk_static finds the library's workspace of this device looked up already
+        void* ws = nullptr;
+        rc = static_scratch(&ws);
+        if (rc) { (void)hipModuleUnload(m->mod); delete m; return rc; }
+    }
     m->persist_grid = 0;
     if (desc->persistent) {
         int per_cu = 0, dev = 0;
@@ -1018,12 +1076,24 @@ int hrn_launch_splitk_static(const hrn_module* mod, const hrn_problem* p, const 
         return fail(HRN_E_BADPARAM, "split-K partial sums of %lld bytes (%d slices x %d x %d x %d x 4) exceed the library's static workspace of %lld bytes",
                     (long long)need, split, p->batch, p->m, p->n, (long long)HRN_STATIC_WORKSPACE_BYTES);
     void* ws = nullptr;
-    int rc = static_scratch(&ws);
+    int dev = 0;
+    int rc = static_scratch(&ws, &dev);
     if (rc) return rc;
     LaunchPlan plan;
     rc = fill_args(mod, p, A, B, C, ws, (size_t)HRN_STATIC_WORKSPACE_BYTES, &plan);
     if (rc) return rc;
-    return run_plan(mod, p, plan, ws, (hipStream_t)stream);
+    // Every call on a GPU shares that GPU's one workspace.  Calls on one stream are ordered by the stream; a call on
+    // another stream is made to wait for the previous user (an event recorded behind each call), so calls from several
+    // streams or threads are serialised on the device instead of racing.
+    hipStream_t st = (hipStream_t)stream;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_used[dev] && g_scratch_stream[dev] != st) HIP_TRY(hipStreamWaitEvent(st, g_scratch_done[dev], 0));
+    rc = run_plan(mod, p, plan, ws, st);
+    if (rc) return rc;
+    HIP_TRY(hipEventRecord(g_scratch_done[dev], st));
+    g_scratch_stream[dev] = st;
+    g_scratch_used[dev] = true;
+    return HRN_OK;
 }
 
 int hrn_time(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, int number, int repeat,

@@ -44,10 +44,21 @@ class perfBuffer:
             out.write(self.encode(sample) + '\n')
         return True
 
+    def record_confirmed(self, sample):
+        """Files the re-timing of a point at the end of a search (long repeats): one more line of records.txt, marked
+        ``"confirmed": true`` - the key the reference's format does not have, and the rows ``Task.apply_best``
+        prefers.  The search's own tables (``perfs``, ``data_x`` / ``data_y``) keep the first measurement."""
+        self.confirmed = getattr(self, "confirmed", {})
+        self.confirmed[sample.stmt_code] = sample.perf
+        with open(os.path.join(self.config.log_dir, self.RECORD_FILE), 'a') as out:
+            out.write(self.encode(sample, confirmed=True) + '\n')
+
     @staticmethod
-    def encode(sample):
+    def encode(sample, confirmed=False):
         row = {"code": sample.stmt_code, "perf": sample.perf, "latency": math.exp(-sample.perf), "time": time.time(),
                "param": sample.knob_manager.solved_knob_vals_phenotype}
+        if confirmed:
+            row["confirmed"] = True
         return json.dumps(row)
 
     def getPerf(self, sample):

@@ -29,9 +29,9 @@ _spawn = mp.get_context("spawn")
 
 
 def _problem_to_dict(p):
-    """The shape fields of an hrn_problem; a split-K workspace is device memory of the process that launches, so
-    the measurement server binds its own."""
-    return {name: int(getattr(p, name)) for name, _ in p._fields_ if name not in ("workspace", "workspace_bytes")}
+    """The shape fields of an hrn_problem; a split-K workspace and column sums are device memory of the process that
+    launches, so the measurement server binds its own."""
+    return {name: int(getattr(p, name)) for name, _ in p._fields_ if name not in ("workspace", "workspace_bytes", "bsum")}
 
 
 def _compile_worker(desc_tuple, timeout_s):

@@ -1,7 +1,7 @@
 """The tuned template instances of the benchmark configurations.
 
 ``tests/quick_start/rocm/tuned/<CASE>/records.txt`` holds the best records of a search on MI355X per case
-(``run.py -c configs/<case>.json``, trimmed with ``keep_best.py``); ``load(name)`` replays the best of them through
+(``run.py -c configs/<case>.json --keep-best N``); ``load(name)`` replays the best of them through
 ``Task.apply_best`` - the same path ``run.py -t`` takes - and returns the template descriptor, its launch-time
 parameters and the record it came from.  The benchmark, smoke and the full-size GPU tests all run these instances.
 """
@@ -50,7 +50,7 @@ def load(name):
     task.config = cfg
     with contextlib.redirect_stdout(io.StringIO()):      # building the template prints the task's arguments
         sched, _ = task.apply_best(path)
-    best = max((json.loads(line) for line in open(path) if line.strip()), key=lambda r: r["perf"])
+    best = Task.best_record(path)
     inst = TunedInstance(name, sched.to_desc(), int(sched.params['group_m']), int(sched.params.get('split_k', 1)),
                          best["code"], math.exp(-best["perf"]), path, dict(sched.params))
     _cache[name] = inst

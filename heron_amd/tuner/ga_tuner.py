@@ -168,6 +168,9 @@ class CGATuner(_ConstrainedGA):
         # load spread, raster group, epilogue kind) move a good tile by a few percent, less than the cost model resolves
         return float(getattr(self.config, 'refine_share', 0.25))
 
+    def confirmation_tiles(self):
+        return int(getattr(self.config, 'confirm_tiles', 8))
+
     def inferKeyVariables(self, env, pop):
         self.key_variables = self._random_keys(env.task)
 

@@ -42,6 +42,11 @@ class Tuner:
         measured points (the constrained GA switches it on); the reference has no such phase."""
         return 0.0
 
+    def confirmation_tiles(self):
+        """Number of distinct block tiles whose best measured points are re-timed, with long repeats, when the search
+        is over (0 = no such phase: the reference has none, and only the constrained GA switches it on)."""
+        return 0
+
     # ------------------------------------------------------------------------------------------------ cost model
     def buildCostModel(self, task):
         self.cost_model = XGBoostCostModel(task, self.config)
@@ -116,7 +121,84 @@ class Tuner:
                 pick = lambda cands, q=quota: self.epsilon_select(env, cands, self.EPSILON, q)   # noqa: E731
             population = self._round(env, iter_no, population, stat, start_time, pick, measure=do_measure,
                                      train=iter_no != len(quotas) - 1)
+        if do_measure and self.confirmation_tiles() > 0:
+            self.confirm(env, self.confirmation_tiles())
         return population, stat
+
+    # ------------------------------------------------------------------------------------------------ confirmation
+    def confirmation_candidates(self, env, tiles):
+        """The best measured point of each of the ``tiles`` best distinct block tiles, plus - for each - the same tile
+        with the wave grid transposed, with the other issue order, and with both: the moves that change a good tile
+        by a few percent, which is what separates one search from the next."""
+        buf = env.perf_buffer
+        order = sorted(range(len(buf.data_y)), key=lambda i: -buf.data_y[i])
+        bases, seen_tiles = [], set()
+        for i in order:
+            sample = buf.samples[i]
+            pheno = sample.knob_manager.solved_knob_vals_phenotype
+            tile = tuple(v for k, v in sorted(pheno.items()) if k.startswith("V#") and k.endswith(("block_m", "block_n")))
+            tile += tuple(v for k, v in sorted(pheno.items()) if k.startswith("P#") and k.endswith("block_k_bytes"))
+            if tile not in seen_tiles:
+                seen_tiles.add(tile)
+                bases.append(sample)
+            if len(bases) >= tiles:
+                break
+        out, seen = [], set()
+
+        def consider(knobs):
+            s = Sample(env.task)
+            point, valid = s.knob_manager.validate(knobs)
+            code = Code(point) if valid else None
+            if valid and code not in seen:
+                seen.add(code)
+                s.point, s.valid, s.stmt_code, s.violation = point, True, code, 0
+                out.append(s)
+
+        for base in bases:
+            geno = base.knob_manager.solved_knob_vals_genotype
+            names = base.knob_manager.knob_names
+            twin = {n: n[:-2] + ("_n" if n.endswith("_m") else "_m") for n in names if n.endswith(("_m", "_n"))}
+            twin = {n: t for n, t in twin.items() if t in geno and not n.endswith("group_m")}
+            order_knob = [n for n in names if n.endswith("issue_order")]
+            for transposed in (False, True):
+                knobs = {n: geno[twin.get(n, n)] for n in names} if (transposed and twin) else dict(geno)
+                consider(dict(knobs))
+                for n in order_knob:
+                    for cand in base.knob_manager.get_knob_candidates(n):
+                        if cand != knobs[n]:
+                            consider(dict(knobs, **{n: cand}))
+        return out
+
+    def confirm(self, env, tiles, min_repeat_ms=100.0, repeat=3):
+        """Deterministic end of a search: every confirmation candidate is timed again with repeats of at least
+        ``min_repeat_ms`` and filed as a confirmed record; ``Task.apply_best`` prefers confirmed records, so the
+        instance a run ships no longer depends on which point a short measurement happened to favour."""
+        cands = self.confirmation_candidates(env, tiles)
+        if not cands:
+            return []
+        print("= ---- Confirmation : %d candidates, repeats of >= %.0f ms ---- =" % (len(cands), min_repeat_ms))
+        from ..runner.measure import MeasureInput
+        from ..runner.runner import perf_of
+        runner = env.runner.measure_option.get('runner') if isinstance(env.runner.measure_option, dict) else None
+        saved = {}
+        for attr, value in (("min_repeat_ms", min_repeat_ms), ("repeat", repeat), ("number", 1)):
+            if runner is not None and hasattr(runner, attr):
+                saved[attr] = getattr(runner, attr)
+                setattr(runner, attr, value)
+        try:
+            task = env.task
+            results = env.runner.measure_batch([MeasureInput(task.target, task, s.knob_manager) for s in cands])
+        finally:
+            for attr, value in saved.items():
+                setattr(runner, attr, value)
+        for sample, result in zip(cands, results):
+            sample.valid, sample.perf = perf_of(result)
+            if sample.valid:
+                env.perf_buffer.record_confirmed(sample)
+        done = sorted((s for s in cands if s.valid), key=lambda s: -s.perf)
+        if done:
+            print("confirmed best %f (latency %.6f ms)" % (done[0].perf, 1e3 * np.exp(-done[0].perf)))
+        return done
 
     def optimize(self, env, population, stat, s_time):
         raise NotImplementedError()

@@ -45,16 +45,20 @@ def DeCode(code):
 
 
 def anaCostModel(model, key_list):
-    """Variable names ordered by the cost model's feature importance (random when untrained)."""
-    bst = model.bst
-    if bst is None:
+    """The variable names of ``key_list`` ordered by how much the cost model relies on each (feature ``f<i>`` of the
+    booster is variable ``i``); variables the trees never split on keep their order behind the ranked ones.  An
+    untrained model ranks nothing: the list is shuffled in place and returned.  Same contract as utils.py:319-332 of
+    the reference."""
+    if model.bst is None:
         random.shuffle(key_list)
         return key_list
-    score_map = bst.get_score(importance_type='weight')
-    score_list_sorted = sorted(score_map.items(), key=lambda x: -x[1])
-    selected_idxs = [int(x[0].split('f')[1]) for x in score_list_sorted]
-    missing = [x for x in range(len(key_list)) if x not in selected_idxs]
-    return [key_list[x] for x in selected_idxs + missing]
+    weight = [0.0] * len(key_list)
+    for name, score in model.bst.get_score(importance_type='weight').items():
+        idx = int(name[1:])
+        if 0 <= idx < len(weight):
+            weight[idx] = float(score)
+    order = sorted(range(len(key_list)), key=lambda i: (weight[i] <= 0.0, -weight[i], i))
+    return [key_list[i] for i in order]
 
 
 def removedot(name):

@@ -196,9 +196,12 @@ int hrn_launch_conv2d_nhwc_u8s8(const hrn_module* mod, const hrn_problem* p, con
  * launching a split_k instance through the entry points above, except that the partial sums go to a workspace that
  * is part of the library's own device image (HRN_STATIC_WORKSPACE_BYTES per GPU, held until the process ends) instead
  * of hrn_problem.workspace, which is ignored.  A problem whose partial sums (slices * batch * m * n * 4 bytes) exceed
- * that size is refused with HRN_E_BADPARAM.  Every call on a GPU uses that GPU's one workspace: calls that overlap
- * in time on one GPU (different streams or threads) race; nothing in it needs to be zero between calls.  Calls no
- * hipMalloc / hipFree.
+ * that size is refused with HRN_E_BADPARAM.  Every call on a GPU uses that GPU's one workspace: a call on another
+ * stream than the previous one first waits (on the device) for that previous call, so calls from several streams or
+ * host threads are serialised rather than racing; nothing in the workspace needs to be zero between calls.  Calls no
+ * hipMalloc / hipFree; the workspace's address and the ordering event are set up by hrn_build of a split_k instance.
+ * The cross-stream wait is an event wait, which a stream under graph capture cannot take from a stream outside the
+ * capture: inside a capture keep to one stream.
  */
 #define HRN_STATIC_WORKSPACE_BYTES (32u << 20)
 int hrn_launch_splitk_static(const hrn_module* mod, const hrn_problem* p, const void* A, const void* B, void* C, void* stream);
@@ -268,6 +271,12 @@ int hrn_probe_launch(int grid, int repeat, double* us_out, void* stream);
  * a kernel that only reads, like the P x V batch_matmul, can draw from HBM when the buffer exceeds the caches. */
 int hrn_probe_read(const void* src, size_t bytes, int repeat, double* gbs_out, void* stream);
 int hrn_probe_mfma(int dtype, int mfma, int random_operands, double* tops_out, void* stream);
+/* hrn_probe_traffic_cold times, `repeat` times, ONE launch of a kernel that reads read_bytes from src and writes
+ * write_bytes to dst (16-byte words, 16 bytes per lane) right after the caches were flushed with flush_buf exactly as
+ * hrn_time_cold does; us_out holds `repeat` microsecond values.  With a workload's algorithmic byte counts this is the
+ * like-for-like floor of its cold launch: same flush, same single dispatch, nothing but the traffic. */
+int hrn_probe_traffic_cold(const void* src, size_t read_bytes, void* dst, size_t write_bytes, void* flush_buf,
+                           size_t flush_bytes, int repeat, double* us_out, void* stream);
 int hrn_probe_copy(const void* src, void* dst, size_t bytes, int repeat, double* gbs_out, void* stream);
 
 /*

@@ -1,4 +1,4 @@
-"""Per-operator experiment:  python run.py [-m trials] [--only f16_gemm,int8_c2d] [-o results.json]
+"""Per-operator experiment:  python run.py [-m trials] [--only f16_gemm,int8_c2d] [--configs DIR] [--check] [-o results.json]
 
 Tunes every case of every configs/*.json (the operator shape lists of the reference's tests/figure6 and tests/figure8
 experiments) with the rocm backend and writes one table of latencies; each config can also be run on its own with
@@ -27,13 +27,16 @@ def main():
     ap.add_argument("-d", "--device_id", type=int, default=0)
     ap.add_argument("--only", default="", help="comma separated config names without .json")
     ap.add_argument("-o", "--out", default="results.json")
+    ap.add_argument("--configs", default=os.path.join(HERE, "configs"), help="directory of case files (default: the shipped lists)")
+    ap.add_argument("--check", action="store_true", help="verify every measured kernel against a host reference "
+                                                         "(gemm, bmm and c2d cases; the measurer reports a mismatch as error 100)")
     args = ap.parse_args()
-    names = sorted(os.path.basename(f)[:-5] for f in glob.glob(os.path.join(HERE, "configs", "*.json")))
+    names = sorted(os.path.basename(f)[:-5] for f in glob.glob(os.path.join(args.configs, "*.json")))
     if args.only:
         names = [n for n in names if n in args.only.split(",")]
     rows = []
     for name in names:
-        args.config = os.path.join(HERE, "configs", name + ".json")
+        args.config = os.path.join(args.configs, name + ".json")
         config = makeConfig(args)
         config.max_trials = min(args.max_trials, config.max_trials)
         config.device_id = args.device_id
@@ -44,7 +47,7 @@ def main():
             config.tuned = ""
             env = Env(option, config)
             print(name, key, op_name, shape, flush=True)
-            latency = run(op_name, key, shape + [config.in_dtype, config.out_dtype], env, runner)
+            latency = run(op_name, key, shape + [config.in_dtype, config.out_dtype], env, runner, args.check)
             rows.append(dict(config=name, case=key, op=op_name, shape=shape, dtype=config.in_dtype, latency_ms=latency))
             with open(args.out, "w") as f:
                 json.dump(rows, f, indent=1)

@@ -70,6 +70,21 @@ def host_reference(op_name):
     return ref
 
 
+def keep_best(src, dst, n):
+    """Writes the rows of a search that are worth keeping to ``dst`` (what ``-t`` and the benchmark later load through
+    Task.apply_best): every row re-timed by the confirmation phase and the ``n`` best of the others, failed
+    measurements dropped."""
+    import json
+    rows = [json.loads(line) for line in open(src) if line.strip()]
+    confirmed = [r for r in rows if r.get("confirmed") and r["perf"] > 0]
+    plain = sorted((r for r in rows if not r.get("confirmed") and r["perf"] > 0), key=lambda r: -r["perf"])[:n]
+    os.makedirs(os.path.dirname(os.path.abspath(dst)), exist_ok=True)
+    with open(dst, "w") as out:
+        for r in plain + sorted(confirmed, key=lambda r: r["perf"]):          # the best confirmed row comes last
+            out.write(json.dumps(r) + "\n")
+    return len(plain) + len(confirmed)
+
+
 def run(op_name, task_name, params, env, runner, check=False):
     config = env.config
     op = config.get_op(op_name)
@@ -106,6 +121,9 @@ if __name__ == '__main__':
     parser.add_argument("--cold", action="store_true",
                         help="time every launch from flushed caches (the runner's enable_cpu_cache_flush of "
                              "tests/quick_start/dlboost/run.py:89-96, on the GPU): for cases bound by HBM traffic")
+    parser.add_argument("--keep-best", type=str, default="", metavar="DIR",
+                        help="after tuning a case, copy its confirmed rows and its 32 best other rows to "
+                             "DIR/<case>/records.txt (the form of the files under tuned/)")
     parser.add_argument("--pretrained-model", type=str, default="",
                         help="attention cost model saved by tests/pretrain/train_model.py: the search is steered by it "
                              "from the first round and it is not re-trained (pretrain/tune_with_pretrained.py)")
@@ -140,6 +158,10 @@ if __name__ == '__main__':
         env = Env(measure_option, config)
         latency = run(op_name, case_keys[i], case + [config.in_dtype, config.out_dtype], env, runner, args.check)
         cases.append([case, latency])
+        if args.keep_best and not args.tuned:
+            kept = keep_best(os.path.join(config.log_dir, 'records.txt'),
+                             os.path.join(args.keep_best, case_keys[i], 'records.txt'), 32)
+            print("kept %d rows of %s under %s" % (kept, case_keys[i], args.keep_best))
     for tup in cases:
         print("Case %s, latency %f ms." % (str(tup[0]), tup[1]))
     runner.close()

@@ -47,6 +47,35 @@ def test_network_driver_two_layers(hrn, tmp_path):
         assert rows and all(row["perf"] > 0 for row in rows)
 
 
+def test_operator_sweep_driver_on_two_case_files(hrn, tmp_path):
+    """tests/ops_sweep/run.py (the counterpart of the reference's tests/figure6/run.py and tests/figure8/run.py) on
+    two small case files, every measured kernel verified: one table row per case, positive latencies, no record of
+    either search marked wrong."""
+    common = {"method": "CGA", "max_trials": 8, "runner_number": 2, "runner_repeat": 3, "runner_timeout": 50,
+              "build_timeout": 50, "pop_num": 24, "select_num": 12, "iter_walks": 2, "parallel_num": 2,
+              "measure_time_per_round": 8, "confirm_tiles": 2}
+    cfgs = tmp_path / "cfgs"
+    cfgs.mkdir()
+    (cfgs / "f16_gemm.json").write_text(json.dumps({"config": dict(common, out_name="OPS/F16_GEMM", in_dtype="float16",
+                                                                   out_dtype="float16",
+                                                                   cases={"G1": ["gemm", [96, 256, 128]]})}))
+    (cfgs / "int8_c2d.json").write_text(json.dumps({"config": dict(common, out_name="OPS/INT8_C2D", in_dtype="int8",
+                                                                   out_dtype="int32",
+                                                                   cases={"C1": ["c2d", [2, 14, 14, 32, 48, 3, 3, 1, 1, 1, "OhwI32o4i"]],
+                                                                          "C2": ["c2d", [1, 9, 9, 16, 16, 1, 1, 1, 0, 1, "OhwI32o4i"]]})}))
+    out = tmp_path / "sweep.json"
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "ops_sweep", "run.py"), "--configs", str(cfgs), "-m", "8",
+                        "--check", "-o", str(out)], cwd=tmp_path, capture_output=True, text=True, timeout=500)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    table = json.load(open(out))
+    assert [(row["config"], row["case"]) for row in table] == [("f16_gemm", "G1"), ("int8_c2d", "C1"), ("int8_c2d", "C2")]
+    assert all(row["latency_ms"] > 0 for row in table) and r.stdout.count("PASS") == 3
+    for rel in ("F16_GEMM/G1", "INT8_C2D/C1", "INT8_C2D/C2"):
+        rows = [json.loads(l) for l in open(tmp_path / "OPS" / rel / "records.txt")]
+        assert rows and all(row["perf"] > 0 for row in rows), rel        # error 100 (wrong result) would give perf 0
+        assert any(row.get("confirmed") for row in rows), rel
+
+
 def _env(tmp_path, method, trials, case=("gemm", [64, 64, 64]), dtype=("int8", "int32")):
     from heron_amd.config import Config
     from heron_amd.environment import Env

@@ -12,6 +12,7 @@ import oracle
 from heron_amd import backend as B
 from heron_amd import hostops, instances
 from heron_amd.ops.rocm import getOpFromName
+from parity_checks import check_f16
 
 pytestmark = pytest.mark.gpu
 REL_TOL = 1e-2
@@ -61,8 +62,7 @@ def check(got, ref, f16):
     got = got.cpu().numpy()
     assert got.shape == ref.shape, (got.shape, ref.shape)
     if f16:
-        scale = float(np.abs(ref).max()) + 1e-30
-        assert float(np.abs(got.astype(np.float64) - ref).max()) / scale <= REL_TOL
+        check_f16(got, ref)                 # tensor-level 1e-2 and the element-wise bound, as in the other suites
     else:
         assert got.dtype == np.int32 and np.array_equal(got, ref)
 

@@ -143,10 +143,12 @@ def test_cga_tuning_loop_writes_reference_format(tmp_path):
     log = env.config.log_dir
     for f in ("schedule.py", "constraints.py", "records.txt", "stat.txt"):
         assert os.path.exists(os.path.join(log, f)), f
-    rows = [json.loads(l) for l in open(os.path.join(log, "records.txt"))]
-    assert 30 <= len(rows) <= 48
-    for r in rows:
-        assert set(r) == {"code", "perf", "latency", "time", "param"}
+    every = [json.loads(l) for l in open(os.path.join(log, "records.txt"))]
+    # the search's own rows carry exactly the reference's keys; the confirmation phase appends rows with one more
+    rows = [r for r in every if not r.get("confirmed")]
+    assert 30 <= len(rows) <= 48 and len(every) > len(rows)
+    for r in every:
+        assert set(r) - {"confirmed"} == {"code", "perf", "latency", "time", "param"}
         assert r["perf"] == 0.0 or abs(r["latency"] - math.exp(-r["perf"])) < 1e-12
         assert len(r["code"].split("_")) - 1 == len(r["param"])
     stat = [l.strip().split(",") for l in open(os.path.join(log, "stat.txt"))]
@@ -159,7 +161,7 @@ def test_cga_tuning_loop_writes_reference_format(tmp_path):
     # apply_best re-instantiates the best record
     t2 = make_env(tmp_path / "again").task
     s, args = t2.apply_best(os.path.join(log, "records.txt"))
-    best_row = max(rows, key=lambda r: r["perf"])
+    best_row = max([r for r in every if r.get("confirmed")], key=lambda r: r["perf"])
     assert s.params['bm'] == best_row["param"]["V#ST:dense,AX:None,VA:block_m"]
     assert "mfma" in t2.getStmt(t2.knob_manager)
     # constraints.py is re-loadable and equals the live constraint system
@@ -393,11 +395,13 @@ TUNED = os.path.join(os.path.dirname(os.path.abspath(__file__)), "quick_start", 
     ("C2D_F16/C1", "c2d", [32, 56, 56, 64, 64, 3, 3, 1, 1, 1], "float16"),
     ("C2D_INT8/C1", "c2d", [32, 56, 56, 64, 64, 3, 3, 1, 1, 1, "OhwI64o4i"], "int8")])
 def test_shipped_tuned_records_reinstantiate(rel, op, shape, dtype):
-    """The records kept for ``run.py -t`` (the 32 best of a search on MI355X per benchmark case) are feasible points of
+    """The records kept for ``run.py -t`` (the 32 best of a search on MI355X per benchmark case and the rows its
+    confirmation phase re-timed) are feasible points of
     today's constraint system and Task.apply_best turns the best of them into a template instance the library accepts."""
     path = os.path.join(TUNED, rel, "records.txt")
     rows = [json.loads(l) for l in open(path)]
-    assert 1 <= len(rows) <= 32 and all(r["perf"] > 0 for r in rows)
+    plain = [r for r in rows if not r.get("confirmed")]
+    assert 1 <= len(plain) <= 32 and all(r["perf"] > 0 for r in rows)
     cfg = Config()
     cfg.codegen_type = 'GPU_MFMA'
     t = Task("t", getOpFromName(op), shape + [dtype, dtype], "rocm")
@@ -407,7 +411,8 @@ def test_shipped_tuned_records_reinstantiate(rel, op, shape, dtype):
         assert t.knob_manager.solver.SATScore(dict(r["param"])) == 0
     s, args = t.apply_best(path)
     assert B.check_desc(s.to_desc()), B.lib().hrn_last_error()
-    best = max(rows, key=lambda r: r["perf"])
+    confirmed = [r for r in rows if r.get("confirmed")]
+    best = max(confirmed or rows, key=lambda r: r["perf"])          # rows re-timed with long repeats take precedence
     stage = s.info['stage_name']
     assert s.params['bm'] == best["param"]["V#ST:%s,AX:None,VA:block_m" % stage]
 
@@ -496,3 +501,70 @@ def test_analytic_estimate_rewards_co_resident_workgroups():
     one_per_cu = analytic_seconds(info, dict(v, lds_bytes=120000))
     four_per_cu = analytic_seconds(info, dict(v, lds_bytes=32768))
     assert four_per_cu <= two_per_cu < one_per_cu        # (two per CU already reach the HBM floor of this shape)
+
+
+def test_confirmation_phase_retimes_the_best_tiles_and_apply_best_prefers_it(tmp_path, capsys):
+    """The constrained GA ends with a deterministic phase: the best point of each of the best distinct block tiles, its
+    transposed wave grid and the other issue order are timed again with long repeats and filed as confirmed records;
+    apply_best then ships the best CONFIRMED row even when a short measurement of another point looked better."""
+    env = make_env(tmp_path, method="CGA", trials=32)
+    env.config.confirm_tiles = 3
+    np.random.seed(5)
+    random.seed(5)
+    env.tune("T1")
+    out = capsys.readouterr().out
+    assert "Confirmation :" in out and "confirmed best" in out
+    path = os.path.join(env.config.log_dir, "records.txt")
+    rows = [json.loads(line) for line in open(path)]
+    confirmed = [r for r in rows if r.get("confirmed")]
+    plain = [r for r in rows if not r.get("confirmed")]
+    assert 24 <= len(plain) <= 32 and 3 <= len(confirmed) <= 12
+    key = lambda r: (r["param"]["V#ST:dense,AX:None,VA:block_m"], r["param"]["V#ST:dense,AX:None,VA:block_n"],
+                     r["param"]["P#ST:dense,AX:None,PA:block_k_bytes"])
+    tiles = {key(r) for r in confirmed}
+    assert len({tuple(sorted(t[:2])) + t[2:] for t in tiles}) <= 3          # (a transposed wave grid transposes a non-square tile)
+    # every confirmed row is a feasible point; the best tiles of the search are among them
+    best_plain = max(plain, key=lambda r: r["perf"])
+    assert key(best_plain) in {key(r) for r in confirmed}
+    # a lucky short measurement does not decide what ships
+    with open(path, "a") as f:
+        lucky = dict(min(plain, key=lambda r: r["perf"]), perf=max(r["perf"] for r in rows) + 1.0)
+        f.write(json.dumps(lucky) + "\n")
+    s, _ = env.task.apply_best(path)
+    best_conf = max(confirmed, key=lambda r: r["perf"])
+    assert s.params['bm'] == best_conf["param"]["V#ST:dense,AX:None,VA:block_m"]
+    assert abs(math.exp(-best_conf["perf"]) - best_conf["latency"]) < 1e-12
+    # without confirmed rows the best row of the file ships, as in the reference
+    only_plain = str(tmp_path / "plain.txt")
+    open(only_plain, "w").write("\n".join(json.dumps(r) for r in plain) + "\n")
+    s2, _ = env.task.apply_best(only_plain)
+    assert s2.params['bm'] == best_plain["param"]["V#ST:dense,AX:None,VA:block_m"]
+    # other tuners have no such phase
+    from heron_amd.tuner.random_tuner import CRandTuner
+    assert CRandTuner(env.config).confirmation_tiles() == 0
+
+
+def test_problem_travels_to_the_measurement_server_without_its_device_pointers():
+    """The builder hands the problem to the measuring process as plain integers; the pointers in it (split-K workspace,
+    caller-supplied column sums) belong to the process that launches and stay behind."""
+    from heron_amd import backend as B
+    from heron_amd.runner import measure_methods as MM
+    d = MM._problem_to_dict(B.gemm_problem(2, 100, 200, 64, 8, split_k=2))
+    assert d['m'] == 100 and d['n'] == 200 and d['k'] == 64 and d['batch'] == 2 and d['split_k'] == 2
+    assert all(isinstance(v, int) for v in d.values())
+    assert not {'workspace', 'workspace_bytes', 'bsum'} & set(d)
+
+
+def test_variable_ranking_follows_the_boosters_feature_weights():
+    from heron_amd.utils import anaCostModel
+
+    class Booster:
+        def get_score(self, importance_type='weight'):
+            return {'f2': 5.0, 'f0': 1.0, 'f3': 5.0}
+
+    class Model:
+        bst = Booster()
+
+    assert anaCostModel(Model, list('abcde')) == ['c', 'd', 'a', 'b', 'e']
+    Model.bst = None
+    assert sorted(anaCostModel(Model, list('abcde'))) == list('abcde')

@@ -51,6 +51,44 @@ def test_static_workspace_matches_caller_workspace(f16, hrn):
     mod.close()
 
 
+def test_static_workspace_allocates_nothing_and_serialises_streams(hrn):
+    """The entry point takes no device memory (the driver's free-memory figure and torch's allocator are unchanged
+    across calls), also for a batched uint8 problem; and two calls issued back to back on two different streams -
+    which share the one workspace - are ordered by the library: both results equal the caller-workspace results."""
+    desc = [d for d in instances.splitk_descs() if d.op == instances.GEMM and d.dtype == instances.U8 and not d.colsum][0]
+    mod = B.Module(desc)
+    rng = np.random.default_rng(3)
+    cases = []
+    for (b, M, K, N, split) in [(3, 200, 2064, 136, 4), (1, 784, 4608, 256, 8)]:
+        A = rng.integers(0, 256, (b, M, K), dtype=np.uint8)
+        Bm = rng.integers(-128, 128, (b, N, K), dtype=np.int8)
+        a, bb = dev(A), dev(Bm)
+        ref = torch.empty((b, M, N), dtype=torch.int32, device="cuda")
+        p = B.gemm_problem(b, M, N, K, 8, split_k=split)
+        mod.launch(p, a.data_ptr(), bb.data_ptr(), ref.data_ptr())
+        out = torch.full((b, M, N), -5, dtype=torch.int32, device="cuda")
+        cases.append((a, bb, out, ref, B.gemm_problem(b, M, N, K, 8, split_k=split), A, Bm))
+    torch.cuda.synchronize()
+    assert np.array_equal(cases[0][3].cpu().numpy(), oracle.bmm_u8s8s32_scalar(cases[0][5], cases[0][6]))
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    for (a, bb, out, ref, q, _, _), st in zip(cases, (s1, s2)):          # the streams' own queues come into being here
+        mod.launch_splitk_static(q, a.data_ptr(), bb.data_ptr(), out.data_ptr(), st.cuda_stream)
+    torch.cuda.synchronize()
+    for c in cases:
+        c[2].fill_(-5)
+    torch.cuda.synchronize()
+    free0, alloc0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for rounds in range(3):
+        for (a, bb, out, ref, q, _, _), st in zip(cases, (s1, s2)):
+            mod.launch_splitk_static(q, a.data_ptr(), bb.data_ptr(), out.data_ptr(), st.cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_allocated() == alloc0
+    assert torch.cuda.memory_reserved() == reserved0
+    for (a, bb, out, ref, q, _, _) in cases:
+        assert torch.equal(out, ref)
+    mod.close()
+
+
 def test_static_workspace_limits(hrn):
     desc = instances.splitk_descs()[0]
     mod = B.Module(desc)
