@@ -222,6 +222,78 @@ def run_probes(torch, B):
     return out
 
 
+def run_prestage(torch, B, reps=200, cold_reps=10):
+    """The library's own passes around the kernel, each timed warm (``reps`` back-to-back launches between two events)
+    and cold (single launches, each after 1 GiB was streamed through the caches), with the algorithmic bytes it moves and
+    the cold floor of exactly that traffic (``hrn_probe_traffic_cold``)."""
+    from heron_amd import instances
+    stream = torch.cuda.current_stream().cuda_stream
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    rows = []
+
+    def timed(name, shape, launch, read_bytes, write_bytes):
+        for _ in range(10):
+            launch()
+        e0.record()
+        for _ in range(reps):
+            launch()
+        e1.record()
+        e1.synchronize()
+        warm_us = e0.elapsed_time(e1) * 1e3 / reps
+        cold = []
+        for _ in range(cold_reps):
+            flush.add_(1)
+            e0.record()
+            launch()
+            e1.record()
+            e1.synchronize()
+            cold.append(e0.elapsed_time(e1) * 1e3)
+        rb, wb = read_bytes - read_bytes % 16, write_bytes - write_bytes % 16
+        psrc = torch.zeros(rb, dtype=torch.uint8, device="cuda")            # buffers of exactly the sizes the probe touches
+        pdst = torch.empty(wb, dtype=torch.uint8, device="cuda")
+        floor = B.probe_traffic_cold(psrc.data_ptr(), rb, pdst.data_ptr(), wb, flush.data_ptr(), flush.numel(), 5, stream)
+        del psrc, pdst
+        cold_us, floor_us = float(sorted(cold)[len(cold) // 2]), float(sorted(floor)[len(floor) // 2])
+        rows.append({"pass": name, "shape": shape, "read_bytes": read_bytes, "write_bytes": write_bytes,
+                     "warm_us": warm_us, "cold_us": cold_us, "floor_us_cold": floor_us,
+                     "warm_GBs": (read_bytes + write_bytes) / warm_us / 1e3,
+                     "cold_GBs": (read_bytes + write_bytes) / cold_us / 1e3})
+
+    # NCW -> NWC activation of the conv1d sweep cases: 16 x 512 channels x 892 positions, fp16
+    src = torch.randn(16, 512, 892, device="cuda").half()
+    dst = torch.empty(16, 892, 512, dtype=torch.float16, device="cuda")
+    timed("hrn_transpose_pad", "16 x (512 x 892) fp16 -> 16 x (892 x 512)",
+          lambda: B.transpose_pad(src.data_ptr(), dst.data_ptr(), 16, 512, 892, 512, 2, stream),
+          src.numel() * 2, dst.numel() * 2)
+    # 3-channel stem -> 8 channels: 16 x 224 x 224 pixels, fp16
+    src2 = torch.randn(16 * 224 * 224, 3, device="cuda").half()
+    dst2 = torch.empty(16 * 224 * 224, 8, dtype=torch.float16, device="cuda")
+    timed("hrn_pad_rows", "802816 pixels x 3 -> 8 channels fp16",
+          lambda: B.pad_rows(src2.data_ptr(), dst2.data_ptr(), 16 * 224 * 224, 3, 8, 2, stream),
+          src2.numel() * 2, dst2.numel() * 2)
+    # column sums of the int8 weight operand of the 8192^3 GEMM
+    src3 = torch.randint(-128, 128, (8192, 8192), dtype=torch.int8, device="cuda")
+    dst3 = torch.empty(8192, dtype=torch.int32, device="cuda")
+    timed("hrn_colsum_s8", "8192 x 8192 int8 -> 8192 int32",
+          lambda: B.colsum_s8(src3.data_ptr(), dst3.data_ptr(), 1, 8192, 8192, stream=stream),
+          src3.numel(), dst3.numel() * 4)
+    # split-K: ResNet-50's 7x7x512 3x3 layer as a GEMM (M = 16*7*7, K = 9*512), 4 slices -> kernel + splitk_reduce_kernel
+    desc = [d for d in instances.splitk_descs() if d.op == instances.GEMM and d.dtype == instances.F16][0]
+    mod = B.Module(desc)
+    M, K, N, split = 784, 4608, 512, 4
+    a = (torch.randn(M, K, device="cuda") * 0.1).half()
+    b = (torch.randn(N, K, device="cuda") * 0.1).half()
+    c = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    prob = B.gemm_problem(1, M, N, K, 8, split_k=split)
+    ws = B.splitk_workspace_bytes(desc, prob)
+    timed("split-K GEMM + splitk_reduce_kernel", "784 x 4608 x 512 fp16, 4 slices (workspace %d bytes)" % ws,
+          lambda: mod.launch(prob, a.data_ptr(), b.data_ptr(), c.data_ptr(), stream),
+          (M * K + N * K) * 2 + ws, M * N * 2 + ws)
+    mod.close()
+    return rows
+
+
 def roofline(w, seconds, workloads):
     """Roofline entry from the algorithmic work / bytes of one launch and its duration."""
     ai = w["ops"] / w["bytes"]
@@ -285,6 +357,9 @@ def main():
     ap.add_argument("--workload", default=HEADLINE)
     ap.add_argument("--only", action="store_true", help="skip the 'also' workloads, the probes and the CPU baseline")
     ap.add_argument("--probe", action="store_true", help="only run the roofline probes (MFMA loop, 1 GiB copy)")
+    ap.add_argument("--prestage", action="store_true",
+                    help="only time the library's passes around the kernel (transpose, channel padding, column sums, "
+                         "split-K reduction), warm and cold")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the hot path is a single-GPU kernel and no multi-GPU figure is produced "
@@ -300,6 +375,9 @@ def main():
     B.lib()
     if args.probe:
         print(json.dumps({"probes": run_probes(torch, B)}))
+        return
+    if args.prestage:
+        print(json.dumps({"prestage": run_prestage(torch, B)}))
         return
     if args.workload not in tuned.CASES:
         print("unknown workload %s (have %s)" % (args.workload, sorted(tuned.CASES)), file=sys.stderr)
