@@ -35,21 +35,39 @@ def records_path(name):
     return os.path.join(TUNED_DIR, CASES[name][0], "records.txt")
 
 
+def instantiate(name, op, shape, dtype, path):
+    """(template schedule, kernel-side argument tensors) of the best record in ``path`` for one case."""
+    from .config import Config
+    from .ops.rocm import getOpFromName
+    from .task.task import Task
+    cfg = Config()
+    cfg.codegen_type, cfg.target_name = 'GPU_MFMA', 'rocm'
+    task = Task(name, getOpFromName(op), list(shape) + [dtype, dtype], "rocm")
+    task.config = cfg
+    with contextlib.redirect_stdout(io.StringIO()):      # building the template prints the task's arguments
+        return task.apply_best(path)
+
+
+def case_file_descs(config_path, tuned_dir):
+    """Descriptors of the best record of every case of a JSON case file that has ``tuned_dir/<case>/records.txt``
+    (the layers of a network, tests/network/configs + tests/network/tuned)."""
+    cfg = json.load(open(config_path))["config"]
+    out = []
+    for name, entry in cfg["cases"].items():
+        path = os.path.join(tuned_dir, name, "records.txt")
+        if os.path.exists(path):
+            out.append(instantiate(name, entry[0], entry[1], cfg["in_dtype"], path)[0].to_desc())
+    return out
+
+
 def load(name):
     """The best record of case ``name`` as a TunedInstance (cached)."""
     if name in _cache:
         return _cache[name]
-    from .config import Config
-    from .ops.rocm import getOpFromName
     from .task.task import Task
     rel, op, shape, dtype = CASES[name]
     path = records_path(name)
-    cfg = Config()
-    cfg.codegen_type, cfg.target_name = 'GPU_MFMA', 'rocm'
-    task = Task(name, getOpFromName(op), shape + [dtype, dtype], "rocm")
-    task.config = cfg
-    with contextlib.redirect_stdout(io.StringIO()):      # building the template prints the task's arguments
-        sched, _ = task.apply_best(path)
+    sched, _ = instantiate(name, op, shape, dtype, path)
     best = Task.best_record(path)
     inst = TunedInstance(name, sched.to_desc(), int(sched.params['group_m']), int(sched.params.get('split_k', 1)),
                          best["code"], math.exp(-best["perf"]), path, dict(sched.params))

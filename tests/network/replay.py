@@ -14,8 +14,6 @@ rounds).  Layers that need an operand adapter (the 3-channel stem) run their ker
 the replay measures kernels and their dispatch, not the Python pre-stage.
 """
 import argparse
-import contextlib
-import io
 import json
 import os
 import sys
@@ -24,19 +22,6 @@ import numpy as np
 
 ROOT = os.path.abspath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", ".."))
 sys.path.insert(0, ROOT)
-
-
-def instantiate(name, op_name, shape, dtype, records):
-    from heron_amd.config import Config
-    from heron_amd.ops.rocm import getOpFromName
-    from heron_amd.task.task import Task
-    cfg = Config()
-    cfg.codegen_type, cfg.target_name = 'GPU_MFMA', 'rocm'
-    task = Task(name, getOpFromName(op_name), shape + [dtype, dtype], "rocm")
-    task.config = cfg
-    with contextlib.redirect_stdout(io.StringIO()):
-        sched, args = task.apply_best(records)
-    return sched, args
 
 
 def main():
@@ -50,6 +35,7 @@ def main():
 
     import torch
     from heron_amd import backend as B
+    from heron_amd import tuned
     if not torch.cuda.is_available():
         print("replay.py needs a GPU", file=sys.stderr)
         sys.exit(1)
@@ -60,7 +46,7 @@ def main():
     layers = []
     for name, (op_name, shape, times) in cfg["cases"].items():
         rec = os.path.join(args.tuned_dir, name, "records.txt")
-        sched, targs = instantiate(name, op_name, list(shape), dtype, rec)
+        sched, targs = tuned.instantiate(name, op_name, list(shape), dtype, rec)
         desc, prob = sched.to_desc(), sched.to_problem()
         mod = B.Module(desc)
         tens = []

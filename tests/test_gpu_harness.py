@@ -76,6 +76,20 @@ def test_operator_sweep_driver_on_two_case_files(hrn, tmp_path):
         assert any(row.get("confirmed") for row in rows), rel
 
 
+def test_network_replay_as_one_stream_and_as_one_graph(hrn, tmp_path):
+    """tests/network/replay.py on the BERT case file: the tuned layers run as one sequence on a stream and from a HIP
+    graph; the driver itself compares every checked graph replay with the eager results and fails on a difference."""
+    net = os.path.join(ROOT, "tests", "network")
+    out = tmp_path / "replay.json"
+    r = subprocess.run([sys.executable, os.path.join(net, "replay.py"), "-c", os.path.join(net, "configs", "bert.json"),
+                        "-T", os.path.join(net, "tuned", "bert"), "--reps", "5", "--rounds", "3", "-o", str(out)],
+                       cwd=tmp_path, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    res = json.load(open(out))
+    assert res["layers"] == 3 and res["launches"] == 84 and res["graph_rounds_checked"] == 3
+    assert 0 < res["graph_us"] < 3 * res["isolated_sum_us"] and 0 < res["stream_us"] < 3 * res["isolated_sum_us"]
+
+
 def _env(tmp_path, method, trials, case=("gemm", [64, 64, 64]), dtype=("int8", "int32")):
     from heron_amd.config import Config
     from heron_amd.environment import Env
