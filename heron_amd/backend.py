@@ -46,6 +46,20 @@ class DevInfo(ctypes.Structure):
         return d
 
 
+GATHER_DIMS = 6
+GATHER_COPY, GATHER_CENTER_SQUARE = 0, 1
+
+
+class Gather(ctypes.Structure):
+    """hrn_gather: the affine index map of one injective pre-stage pass."""
+    _fields_ = [("ndim", ctypes.c_int32), ("nsrc", ctypes.c_int32), ("elem_bytes", ctypes.c_int32), ("op", ctypes.c_int32),
+                ("reserved", ctypes.c_int32 * 2),
+                ("dst_dim", ctypes.c_int64 * GATHER_DIMS), ("dst_stride", ctypes.c_int64 * GATHER_DIMS),
+                ("dst_live", ctypes.c_int64 * GATHER_DIMS), ("src_dim", ctypes.c_int64 * GATHER_DIMS),
+                ("src_stride", ctypes.c_int64 * GATHER_DIMS), ("add", ctypes.c_int64 * GATHER_DIMS),
+                ("div", ctypes.c_int64 * GATHER_DIMS), ("mul", (ctypes.c_int64 * GATHER_DIMS) * GATHER_DIMS)]
+
+
 class KernelDesc(ctypes.Structure):
     _fields_ = [("dtype", ctypes.c_int32), ("op", ctypes.c_int32), ("bm", ctypes.c_int32), ("bn", ctypes.c_int32),
                 ("bkb", ctypes.c_int32), ("wm", ctypes.c_int32), ("wn", ctypes.c_int32), ("mfma", ctypes.c_int32),
@@ -148,6 +162,7 @@ SYMBOLS = {
     "hrn_pad_rows": (_i, [_vp, _vp, ctypes.c_size_t, _i, _i, _i, _vp]),
     "hrn_colsum_s8": (_i, [_vp, _vp, _i, _i, _i, _i, ctypes.c_int64, _vp]),
     "hrn_transpose_pad": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "hrn_gather_nd": (_i, [ctypes.POINTER(Gather), _vp, _vp, _vp, _vp]),
     "hrn_probe_read": (_i, [_vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_probe_traffic_cold": (_i, [_vp, ctypes.c_size_t, _vp, ctypes.c_size_t, _vp, ctypes.c_size_t, _i, ctypes.POINTER(_d), _vp]),
     "hrn_last_error": (ctypes.c_char_p, []),
@@ -262,6 +277,36 @@ def pad_rows(src_ptr, dst_ptr, rows, c, cp, elem_bytes, stream=0):
 def transpose_pad(src_ptr, dst_ptr, batch, rows, cols, rows_padded, elem_bytes, stream=0):
     """dst[b][c][r] = src[b][r][c], rows of dst zero-padded to rows_padded (device pointers)."""
     _check(lib().hrn_transpose_pad(src_ptr, dst_ptr, batch, rows, cols, rows_padded, elem_bytes, stream))
+
+
+def make_gather(elem_bytes, dst_dim, src, dst_stride=None, dst_live=None, op=GATHER_COPY):
+    """Builds an hrn_gather.  ``dst_dim``: extents of dst (outermost first; contiguous unless ``dst_stride`` is given);
+    ``src``: one entry per source coordinate, ``(extent, stride, {dst dimension: multiplier}, add, div)`` with ``add`` and
+    ``div`` optional (0 and 1): coordinate = (add + sum multiplier * index) / div."""
+    g = Gather()
+    nd, ns = len(dst_dim), len(src)
+    if not (1 <= nd <= GATHER_DIMS and 1 <= ns <= GATHER_DIMS):
+        raise ValueError("a gather has 1..%d dst dimensions and source coordinates" % GATHER_DIMS)
+    g.ndim, g.nsrc, g.elem_bytes, g.op = nd, ns, int(elem_bytes), int(op)
+    stride = 1
+    for d in range(nd - 1, -1, -1):
+        g.dst_dim[d] = int(dst_dim[d])
+        g.dst_stride[d] = int(dst_stride[d]) if dst_stride is not None else stride
+        g.dst_live[d] = int(dst_live[d]) if dst_live is not None else int(dst_dim[d])
+        stride *= int(dst_dim[d])
+    for s, entry in enumerate(src):
+        extent, sstride, muls = entry[0], entry[1], entry[2]
+        g.src_dim[s], g.src_stride[s] = int(extent), int(sstride)
+        g.add[s] = int(entry[3]) if len(entry) > 3 else 0
+        g.div[s] = int(entry[4]) if len(entry) > 4 else 1
+        for d, m in muls.items():
+            g.mul[s][d] = int(m)
+    return g
+
+
+def gather_nd(g, src_ptr, dst_ptr, aux_ptr=None, stream=0):
+    """dst = f(gather(src)) as one pass of the library (device pointers; see hrn_gather in the header)."""
+    _check(lib().hrn_gather_nd(ctypes.byref(g), src_ptr, aux_ptr, dst_ptr, stream))
 
 
 def probe_read(src_ptr, nbytes, repeat=10, stream=0):

@@ -682,6 +682,80 @@ __global__ void __launch_bounds__(256) pad_rows_kernel(const unsigned char* __re
     }
 }
 
+// Affine gather (hrn_gather_nd): one lane per 16-byte piece of the innermost dst dimension (VEC) or per element.
+template <int ES, bool VEC, typename IDX>
+__global__ void __launch_bounds__(256) gather_nd_kernel(const hrn_gather g, const char* __restrict__ src,
+                                                        const _Float16* __restrict__ aux, char* __restrict__ dst, IDX total) {
+    const IDX t = (IDX)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    constexpr int V = VEC ? 16 / ES : 1;
+    int64_t idx[HRN_GATHER_DIMS];
+    IDX rem = t;
+#pragma unroll
+    for (int d = HRN_GATHER_DIMS - 1; d >= 0; --d) {
+        idx[d] = 0;
+        if (d < g.ndim) {
+            const IDX ext = (IDX)(d == g.ndim - 1 ? g.dst_dim[d] / V : g.dst_dim[d]);
+            const IDX q = rem / ext;
+            idx[d] = (int64_t)(rem - q * ext) * (d == g.ndim - 1 ? V : 1);
+            rem = q;
+        }
+    }
+    int64_t doff = 0;
+    bool live = true;
+#pragma unroll
+    for (int d = 0; d < HRN_GATHER_DIMS; ++d)
+        if (d < g.ndim) {
+            doff += idx[d] * g.dst_stride[d];
+            live = live && idx[d] < g.dst_live[d];
+        }
+    int64_t soff = 0;
+#pragma unroll
+    for (int s = 0; s < HRN_GATHER_DIMS; ++s)
+        if (s < g.nsrc) {
+            int64_t num = g.add[s];
+#pragma unroll
+            for (int d = 0; d < HRN_GATHER_DIMS; ++d)
+                if (d < g.ndim) num += g.mul[s][d] * idx[d];
+            const int64_t q = num / g.div[s];
+            live = live && num >= 0 && q * g.div[s] == num && q < g.src_dim[s];
+            soff += q * g.src_stride[s];
+        }
+    if constexpr (VEC) {
+        pv4i v = {0, 0, 0, 0};
+        if (live) {
+            v = *(const pv4i*)(src + soff * ES);
+            if (g.op == HRN_GATHER_CENTER_SQUARE) {
+                const pv4i y = *(const pv4i*)((const char*)aux + soff * ES);
+                _Float16 h[8], m[8];
+                __builtin_memcpy(h, &v, 16);
+                __builtin_memcpy(m, &y, 16);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const _Float16 dlt = h[e] - m[e];
+                    h[e] = dlt * dlt;
+                }
+                __builtin_memcpy(&v, h, 16);
+            }
+        }
+        *(pv4i*)(dst + doff * ES) = v;
+    } else if constexpr (ES == 2) {
+        unsigned short v = 0;
+        if (live) {
+            v = *(const unsigned short*)(src + soff * 2);
+            if (g.op == HRN_GATHER_CENTER_SQUARE) {
+                const _Float16 dlt = __builtin_bit_cast(_Float16, v) - aux[soff];
+                v = __builtin_bit_cast(unsigned short, (_Float16)(dlt * dlt));
+            }
+        }
+        *(unsigned short*)(dst + doff * 2) = v;
+    } else if constexpr (ES == 1) {
+        dst[doff] = live ? src[soff] : (char)0;
+    } else {
+        *(unsigned int*)(dst + doff * 4) = live ? *(const unsigned int*)(src + soff * 4) : 0u;
+    }
+}
+
 // Batched transpose src[b][r][c] -> dst[b][c][r'] with r' padded to rp >= rows (zeros), through a 64x64 LDS tile so that
 // both the reads (along c) and the writes (along r) are contiguous.  blockDim = (64, 4).
 template <typename T>
@@ -781,6 +855,72 @@ int hrn_transpose_pad(const void* src, void* dst, int batch, int rows, int cols,
     else transpose_pad_kernel<unsigned int><<<grid, block, 0, st>>>((const unsigned int*)src, (unsigned int*)dst, rows, cols, rows_padded);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HRN_E_LAUNCH, "transpose_pad: %s", hipGetErrorString(e));
+    return HRN_OK;
+}
+
+int hrn_gather_nd(const hrn_gather* g, const void* src, const void* aux, void* dst, void* stream) {
+    if (!g || !src || !dst) return fail(HRN_E_BADPARAM, "gather: null argument");
+    const int nd = g->ndim, ns = g->nsrc, es = g->elem_bytes;
+    if (nd < 1 || nd > HRN_GATHER_DIMS || ns < 1 || ns > HRN_GATHER_DIMS || (es != 1 && es != 2 && es != 4))
+        return fail(HRN_E_BADPARAM, "gather: %d dst dimensions, %d source coordinates, %d-byte elements", nd, ns, es);
+    if (g->op != HRN_GATHER_COPY && g->op != HRN_GATHER_CENTER_SQUARE)
+        return fail(HRN_E_BADPARAM, "gather: unknown op %d", g->op);
+    if (g->op == HRN_GATHER_CENTER_SQUARE && (es != 2 || !aux))
+        return fail(HRN_E_BADPARAM, "gather: center-square takes fp16 elements and an aux tensor laid out like src");
+    if (g->dst_stride[nd - 1] != 1) return fail(HRN_E_BADPARAM, "gather: the innermost dst dimension must have stride 1");
+    // the largest dst and src offsets any index can reach; totals that overflow are refused
+    long double total_ld = 1, dmax = 0, smax = 0;
+    for (int d = 0; d < nd; ++d) {
+        if (g->dst_dim[d] < 0 || g->dst_stride[d] < 0 || g->dst_live[d] < 0 || g->dst_live[d] > g->dst_dim[d])
+            return fail(HRN_E_BADPARAM, "gather: dst dimension %d: extent %lld, stride %lld, live %lld", d, (long long)g->dst_dim[d],
+                        (long long)g->dst_stride[d], (long long)g->dst_live[d]);
+        total_ld *= (long double)g->dst_dim[d];
+        dmax += (long double)(g->dst_dim[d] ? g->dst_dim[d] - 1 : 0) * (long double)g->dst_stride[d];
+    }
+    for (int s = 0; s < ns; ++s) {
+        if (g->src_dim[s] < 1 || g->src_stride[s] < 0 || g->div[s] < 1)
+            return fail(HRN_E_BADPARAM, "gather: source coordinate %d: extent %lld, stride %lld, divisor %lld", s, (long long)g->src_dim[s],
+                        (long long)g->src_stride[s], (long long)g->div[s]);
+        smax += (long double)(g->src_dim[s] - 1) * (long double)g->src_stride[s];
+    }
+    if (total_ld > 9.0e15L || dmax > 9.0e15L || smax > 9.0e15L) return fail(HRN_E_BADPARAM, "gather: extents too large");
+    const int64_t total = (int64_t)total_ld;
+    if (total == 0) return HRN_OK;
+    // 16 bytes per lane when whole aligned pieces move along the innermost dimension
+    const int V = 16 / es, d0 = nd - 1;
+    bool vec = g->dst_dim[d0] % V == 0 && g->dst_live[d0] % V == 0 && ((uintptr_t)src % 16) == 0 && ((uintptr_t)dst % 16) == 0 &&
+               (g->op != HRN_GATHER_CENTER_SQUARE || ((uintptr_t)aux % 16) == 0);
+    for (int d = 0; d < d0 && vec; ++d) vec = g->dst_stride[d] % V == 0;
+    int s0 = -1;
+    for (int s = 0; s < ns && vec; ++s) {
+        if (g->mul[s][d0] == 0) {
+            vec = g->src_stride[s] % V == 0;
+            continue;
+        }
+        vec = s0 < 0 && g->mul[s][d0] == 1 && g->div[s] == 1 && g->src_stride[s] == 1 && g->src_dim[s] % V == 0 && g->add[s] % V == 0;
+        for (int d = 0; d < d0 && vec; ++d) vec = g->mul[s][d] % V == 0;
+        s0 = s;
+    }
+    vec = vec && s0 >= 0;
+    const int64_t lanes = vec ? total / V : total;
+    const int64_t blocks = (lanes + 255) / 256;
+    if (blocks > 0x7fffffffLL) return fail(HRN_E_BADPARAM, "gather: %lld elements are more than one launch covers", (long long)total);
+    hipStream_t st = (hipStream_t)stream;
+    const char* sp = (const char*)src;
+    const _Float16* ap = (const _Float16*)aux;
+    char* dp = (char*)dst;
+    const bool small = lanes < (1LL << 31) && total < (1LL << 31);
+#define HRN_GATHER_LAUNCH(ES_, VEC_)                                                                                          \
+    do {                                                                                                                      \
+        if (small) gather_nd_kernel<ES_, VEC_, uint32_t><<<(unsigned)blocks, 256, 0, st>>>(*g, sp, ap, dp, (uint32_t)lanes);   \
+        else gather_nd_kernel<ES_, VEC_, uint64_t><<<(unsigned)blocks, 256, 0, st>>>(*g, sp, ap, dp, (uint64_t)lanes);         \
+    } while (0)
+    if (es == 1) { if (vec) HRN_GATHER_LAUNCH(1, true); else HRN_GATHER_LAUNCH(1, false); }
+    else if (es == 2) { if (vec) HRN_GATHER_LAUNCH(2, true); else HRN_GATHER_LAUNCH(2, false); }
+    else { if (vec) HRN_GATHER_LAUNCH(4, true); else HRN_GATHER_LAUNCH(4, false); }
+#undef HRN_GATHER_LAUNCH
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HRN_E_LAUNCH, "gather: %s", hipGetErrorString(e));
     return HRN_OK;
 }
 

@@ -108,6 +108,14 @@ def _native_ok(t):
     return t.is_cuda and t.is_contiguous() and t.element_size() in (1, 2, 4)
 
 
+def _gather(src, out, dst_dim, coords, dst_stride=None, dst_live=None, op=B.GATHER_COPY, aux=None):
+    """One pass of the library's affine gather from ``src`` into ``out`` (both contiguous device tensors; see
+    backend.make_gather for ``coords``)."""
+    g = B.make_gather(src.element_size(), dst_dim, coords, dst_stride, dst_live, op)
+    B.gather_nd(g, src.data_ptr(), out.data_ptr(), aux.data_ptr() if aux is not None else None, _stream())
+    return out
+
+
 def _channels_last(x3, cp=None):
     """(N, C, L) -> (N, L, cp): channels become the last axis, zero-padded to ``cp`` (one pass of the library)."""
     N, C, L = x3.shape
@@ -160,9 +168,23 @@ def _const_scan(info, A):
     return T
 
 
-def _act_mean(info, In, *_):
+def _channel_major(info, In, mean=None):
+    """(N,C,H,W) -> (C, K) with K = N*H*W zero-padded to the kernel's K; with ``mean`` (same shape as ``In``) every
+    element becomes (x - mean)^2 on the way (fp16, both steps rounded as separate fp16 tensor operations would)."""
     N, C, H, W = In.shape
-    return _pad_last(In.permute(1, 0, 2, 3).reshape(C, N * H * W), info['gemm_view']['K'])
+    K = info['gemm_view']['K']
+    if not (_native_ok(In) and (mean is None or (_native_ok(mean) and In.dtype == torch.float16))):
+        if mean is not None:
+            d = In - mean
+            In = d * d
+        return _pad_last(In.permute(1, 0, 2, 3).reshape(C, N * H * W), K)
+    out = (torch.empty if K == N * H * W else torch.zeros)((C, K), dtype=In.dtype, device=In.device)
+    return _gather(In, out, (C, N, H * W), [(N, C * H * W, {1: 1}), (C, H * W, {0: 1}), (H * W, 1, {2: 1})],
+                   dst_stride=(K, H * W, 1), op=B.GATHER_CENTER_SQUARE if mean is not None else B.GATHER_COPY, aux=mean)
+
+
+def _act_mean(info, In, *_):
+    return _channel_major(info, In)
 
 
 def _const_mean(info, In, *_):
@@ -174,8 +196,9 @@ def _const_mean(info, In, *_):
 
 
 def _act_var(info, In, Mean):
-    d = In - Mean
-    return _act_mean(info, d * d)
+    if tuple(Mean.shape) != tuple(In.shape) or Mean.dtype != In.dtype:
+        raise ValueError("var takes a Mean of In's shape and type, got %s for %s" % (tuple(Mean.shape), tuple(In.shape)))
+    return _channel_major(info, In, Mean)
 
 
 def _cpad(info):
@@ -224,6 +247,12 @@ def _act_c3d_ndhwc(info, X, F):           # (N,D,H,W,CI)
     N, D, H, W, CI = X.shape
     KD, DO, sd, pd, dd = dp['KD'], dp['DO'], dp['stride'], dp['pad'], dp['dil']
     cip = info['conv']['CI'] // KD
+    if _native_ok(X):
+        # depth taps side by side on the channel axis: channel block kd of output slice z is input slice z*sd + kd*dd - pd
+        out = torch.empty((N * DO, H, W, KD * cip), dtype=X.dtype, device=X.device)
+        return _gather(X, out, (N, DO, H * W, KD, cip),
+                       [(N, D * H * W * CI, {0: 1}), (D, H * W * CI, {1: sd, 3: dd}, -pd), (H * W, CI, {2: 1}), (CI, 1, {4: 1})],
+                       dst_live=(N, DO, H * W, KD, CI))
     Xp = torch.zeros((N, D + 2 * pd, H, W, cip), dtype=X.dtype, device=X.device)
     Xp[:, pd:pd + D, :, :, :CI] = X
     # depth taps side by side on the channel axis: channel block kd of output slice z is input slice z*sd + kd*dd
@@ -254,6 +283,14 @@ def _act_t2d_nchw(info, X, F):            # (N,CI,H,W): zero-expanded by the str
     s = t['stride']
     top = (c['KH'] - 1) * t['dil'] - t['pad']
     left = (c['KW'] - 1) * t['dil'] - t['pad']
+    if _native_ok(X) and N <= 65535:
+        # channels last (and padded) first, then one pass that writes every pixel of the expanded image: input pixel
+        # ((y - top) / s, (x - left) / s) where both divide, zero elsewhere
+        Xc = _channels_last(X.reshape(N, CI, H * W), c['CI'])
+        Xe = torch.empty((N, c['H'], c['W'], c['CI']), dtype=X.dtype, device=X.device)
+        return _gather(Xc, Xe, (N, c['H'], c['W'], c['CI']),
+                       [(N, H * W * c['CI'], {0: 1}), (H, W * c['CI'], {1: 1}, -top, s), (W, c['CI'], {2: 1}, -left, s),
+                        (c['CI'], 1, {3: 1})])
     Xe = torch.zeros((N, c['H'], c['W'], c['CI']), dtype=X.dtype, device=X.device)
     if s > 1:
         # channels last (and padded) first, so that the strided scatter moves whole pixels (stride 2: 137 -> 70 us end
@@ -269,6 +306,11 @@ def _act_dep(info, X, F):                 # (N,C,H,W): the 3x3 windows as 4x4 = 
     d = info['dep']
     N, C, H, W = X.shape
     s, p, HO, WO = d['stride'], d['pad'], d['HO'], d['WO']
+    if _native_ok(X):
+        A = torch.empty((C, N * HO * WO, 16), dtype=X.dtype, device=X.device)
+        return _gather(X, A, (C, N, HO, WO, 4, 4),
+                       [(N, C * H * W, {1: 1}), (C, H * W, {0: 1}), (H, W, {2: s, 4: 1}, -p), (W, 1, {3: s, 5: 1}, -p)],
+                       dst_live=(C, N, HO, WO, 3, 3))
     Xp = torch.zeros((N, C, H + 2 * p + 1, W + 2 * p + 1), dtype=X.dtype, device=X.device)
     Xp[:, :, p:p + H, p:p + W] = X
     A = torch.zeros((C, N, HO, WO, 4, 4), dtype=X.dtype, device=X.device)
@@ -288,6 +330,10 @@ def _const_dep(info, X, F):               # (K,3,3)
 
 def _fin_dep(info, Cm):                   # (C, N*HO*WO, NP) -> (N, C, NP, HO, WO)
     d = info['dep']
+    C, N, HW, NP = d['C'], d['N'], d['HO'] * d['WO'], d['NP']
+    if _native_ok(Cm):
+        out = torch.empty((N, C, NP, d['HO'], d['WO']), dtype=Cm.dtype, device=Cm.device)
+        return _gather(Cm, out, (N, C, NP, HW), [(C, N * HW * NP, {1: 1}), (N, HW * NP, {0: 1}), (HW, NP, {3: 1}), (NP, 1, {2: 1})])
     return Cm.reshape(d['C'], d['N'], d['HO'], d['WO'], d['NP']).permute(1, 0, 4, 2, 3).contiguous()
 
 

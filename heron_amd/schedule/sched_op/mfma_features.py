@@ -110,3 +110,37 @@ def view_of_values(info, values):
 def prior_score(info, values):
     """ln(1 / estimated seconds): comparable to the measured ``perf`` of a sample."""
     return featurize(info, values)[-1]
+
+
+def coupled_moves(names, values, candidates):
+    """Knob assignments a few coordinated steps away from ``values`` that no one-knob change reaches, for the search's
+    refinement rounds: (a) the other MFMA edge at the same block tile (tile counts rescaled), (b) another number of
+    K bytes per LDS row with every stage count (what fits is decided by the constraint system), each with every LDS
+    swizzle, since the conflict-free swizzle depends on both.  ``names``: the task's knob names; ``values``: knob name ->
+    value of the incumbent; ``candidates(name)``: that knob's value list.  Returns (label, knob dictionary) pairs; moves
+    with the same label differ only in the dependent choices (stages, swizzle)."""
+    by = {}
+    for n in names:
+        for k in KNOBS:
+            if n.endswith("PA:" + k) or n.endswith(":" + k):
+                by[k] = n
+    need = ('mfma', 'tile_m', 'tile_n', 'block_k_bytes', 'lds_stages', 'lds_swizzle')
+    if any(k not in by for k in need):
+        return []
+    out = []
+    swizzles = list(candidates(by['lds_swizzle']))
+    mfma, tm, tn = values[by['mfma']], values[by['tile_m']], values[by['tile_n']]
+    for other in candidates(by['mfma']):
+        if other == mfma or (tm * mfma) % other or (tn * mfma) % other:
+            continue
+        for swz in swizzles:
+            out.append(("mfma=%d" % other, dict(values, **{by['mfma']: other, by['tile_m']: tm * mfma // other,
+                                                           by['tile_n']: tn * mfma // other, by['lds_swizzle']: swz})))
+    for bkb in candidates(by['block_k_bytes']):
+        if bkb == values[by['block_k_bytes']]:
+            continue
+        for stages in candidates(by['lds_stages']):
+            for swz in swizzles:
+                out.append(("block_k_bytes=%d" % bkb,
+                            dict(values, **{by['block_k_bytes']: bkb, by['lds_stages']: stages, by['lds_swizzle']: swz})))
+    return out

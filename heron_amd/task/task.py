@@ -117,6 +117,17 @@ class Task:
         info = self.template_info if own_shape else view_of_values(self.template_info, values)
         return featurize(info, values)
 
+    def coupled_moves(self, knob_manager):
+        """(label, knob dictionary) pairs a few coordinated knob changes away from the point ``knob_manager`` holds
+        (operator specific; empty when the operator set defines none); moves that share a label differ only in dependent
+        choices.  Used by the refinement rounds and the confirmation phase of the search."""
+        if self.template_info is None or self.config is None or self.config.codegen_type != 'GPU_MFMA':
+            return []
+        from ..schedule.sched_op.mfma_features import coupled_moves
+        names = list(knob_manager.knob_names)
+        values = {n: knob_manager.solved_knob_vals_genotype[n] for n in names}
+        return coupled_moves(names, values, knob_manager.get_knob_candidates)
+
     # ------------------------------------------------------------------ verification and text form
     def set_verify_func(self, func, rtol=0.1):
         self.rtol = rtol

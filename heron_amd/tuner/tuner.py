@@ -129,7 +129,9 @@ class Tuner:
     def confirmation_candidates(self, env, tiles):
         """The best measured point of each of the ``tiles`` best distinct block tiles, plus - for each - the same tile
         with the wave grid transposed, with the other issue order, and with both: the moves that change a good tile
-        by a few percent, which is what separates one search from the next."""
+        by a few percent, which is what separates one search from the next - and the best-predicted variant of each of
+        the operator's coupled moves.  The best rows of the records files named
+        in ``config.incumbents`` (three confirmed, three others per file) join them."""
         buf = env.perf_buffer
         order = sorted(range(len(buf.data_y)), key=lambda i: -buf.data_y[i])
         bases, seen_tiles = [], set()
@@ -154,6 +156,19 @@ class Tuner:
                 s.point, s.valid, s.stmt_code, s.violation = point, True, code, 0
                 out.append(s)
 
+        # incumbents of earlier searches (config.incumbents: records files) are re-timed under the same conditions,
+        # so a run can only ship something worse than an earlier one if it measures worse today
+        probe = Sample(env.task).knob_manager
+        for path in getattr(self.config, 'incumbents', None) or []:
+            try:
+                rows = [json.loads(line) for line in open(path) if line.strip()]
+            except OSError:
+                print("no incumbents at %s" % path)
+                continue
+            good = sorted((r for r in rows if r.get("perf", 0) > 0), key=lambda r: -r["perf"])
+            for row in [r for r in good if r.get("confirmed")][:3] + [r for r in good if not r.get("confirmed")][:3]:
+                consider({n: row["param"].get(n, probe.solver.vals[n].defv) for n in probe.knob_names})
+
         for base in bases:
             geno = base.knob_manager.solved_knob_vals_genotype
             names = base.knob_manager.knob_names
@@ -167,6 +182,20 @@ class Tuner:
                     for cand in base.knob_manager.get_knob_candidates(n):
                         if cand != knobs[n]:
                             consider(dict(knobs, **{n: cand}))
+            # the operator's coupled moves (other MFMA edge, other LDS row length at the same block tile): of each kind
+            # the feasible variant the cost model likes best, so that a population that settled on the wrong side of a
+            # coarse choice still has the other side timed
+            moves = getattr(env.task, 'coupled_moves', None)
+            groups = {}
+            for label, knobs in (moves(base.knob_manager) if moves else []):
+                s = Sample(env.task)
+                point, valid = s.knob_manager.validate(knobs)
+                if valid:
+                    s.point, s.valid, s.stmt_code, s.violation = point, True, Code(point), 0
+                    groups.setdefault(label, []).append((s, knobs))
+            for label, members in groups.items():
+                self._assign_predictions([m[0] for m in members])
+                consider(max(members, key=lambda m: m[0].predict)[1])
         return out
 
     def confirm(self, env, tiles, min_repeat_ms=100.0, repeat=3):
@@ -259,6 +288,11 @@ class Tuner:
             twin = {n: t for n, t in twin.items() if t in geno and not n.endswith("group_m")}
             if twin:
                 consider({n: geno[twin.get(n, n)] for n in names})
+            # and the operator's own coupled moves (other MFMA edge at the same block tile, other LDS row length with
+            # every stage count): the coarse choices a population can settle on the wrong side of
+            moves = getattr(env.task, 'coupled_moves', None)
+            for _, knobs in (moves(base.knob_manager) if moves else []):
+                consider(knobs)
         return self._assign_predictions(out)
 
     # ------------------------------------------------------------------------------------------------ feasibility table

@@ -256,6 +256,46 @@ int hrn_pad_rows(const void* src, void* dst, size_t rows, int c, int cp, int ele
 int hrn_transpose_pad(const void* src, void* dst, int batch, int rows, int cols, int rows_padded, int elem_bytes, void* stream);
 
 /*
+ * Injective pre-stage as one pass: dst = f(gather(src)).  The reference declares such stages as tensor expressions in
+ * front of its tensorized product and inlines them into the shared-memory load (utils.py:290-303 traverse_inline,
+ * schedule/sched_op/sched_common.py:198-202): zero padding and depth unfolding of conv3d (ops/cuda/conv3d.py), the
+ * stride expansion of the transposed conv (ops/cuda/conv2d_transposed.py:93-104), the 3x3 window gathering of the
+ * depthwise conv (ops/cuda/dep.py), the channel-major view of mean (ops/cuda/mean.py) and (x - mean)^2 of var
+ * (ops/cuda/var.py:9-14).  Here the stage is described by an affine index map and runs as a kernel of the library in
+ * front of hrn_mfma_kernel.
+ *
+ * dst has `ndim` dimensions (outermost first) with extents dst_dim and element strides dst_stride (innermost 1).  For
+ * the element at index (i_0 .. i_{ndim-1}) source coordinate s (0 <= s < nsrc) is
+ *     c_s = (add[s] + sum_d mul[s][d] * i_d) / div[s]
+ * and the element is src[sum_s c_s * src_stride[s]] when every i_d < dst_live[d], every numerator is non-negative and
+ * divisible by div[s] and every c_s < src_dim[s]; otherwise it is zero.  op HRN_GATHER_CENTER_SQUARE (fp16 only) stores
+ * (x - y)^2, both steps rounded to fp16, where a plain copy stores x; y is the element of `aux` at x's offset (aux has
+ * the layout of src: var's Mean operand, ops/cuda/var.py:7-13).  When the innermost dimension
+ * moves whole, aligned 16-byte pieces (the library checks the map, the extents and both pointers) every lane moves 16
+ * bytes, otherwise one element.  All buffers are caller-owned device memory; elements not covered by dst_dim /
+ * dst_stride (row padding) are left alone.
+ */
+#define HRN_GATHER_DIMS 6
+#define HRN_GATHER_COPY 0
+#define HRN_GATHER_CENTER_SQUARE 1
+typedef struct hrn_gather {
+    int32_t ndim;
+    int32_t nsrc;
+    int32_t elem_bytes;       /* 1, 2 or 4 */
+    int32_t op;
+    int32_t reserved[2];
+    int64_t dst_dim[HRN_GATHER_DIMS];
+    int64_t dst_stride[HRN_GATHER_DIMS];
+    int64_t dst_live[HRN_GATHER_DIMS];
+    int64_t src_dim[HRN_GATHER_DIMS];
+    int64_t src_stride[HRN_GATHER_DIMS];
+    int64_t add[HRN_GATHER_DIMS];
+    int64_t div[HRN_GATHER_DIMS];
+    int64_t mul[HRN_GATHER_DIMS][HRN_GATHER_DIMS];   /* mul[s][d] */
+} hrn_gather;
+int hrn_gather_nd(const hrn_gather* g, const void* src, const void* aux, void* dst, void* stream);
+
+/*
  * Roofline probes (no counterpart in the reference, which never relates a timing to a hardware
  * limit).  hrn_probe_mfma times a register-resident loop of independent MFMAs of the given
  * dtype/shape on every CU and returns dense T(FL)OP/s (random_operands != 0 feeds operands with the

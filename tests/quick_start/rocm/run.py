@@ -124,6 +124,9 @@ if __name__ == '__main__':
     parser.add_argument("--keep-best", type=str, default="", metavar="DIR",
                         help="after tuning a case, copy its confirmed rows and its 32 best other rows to "
                              "DIR/<case>/records.txt (the form of the files under tuned/)")
+    parser.add_argument("--incumbents", type=str, default="", metavar="DIR",
+                        help="DIR/<case>/records.txt of earlier searches (the layout --keep-best writes): their best rows "
+                             "are timed again in the confirmation phase, beside this search's own best tiles")
     parser.add_argument("--pretrained-model", type=str, default="",
                         help="attention cost model saved by tests/pretrain/train_model.py: the search is steered by it "
                              "from the first round and it is not re-trained (pretrain/tune_with_pretrained.py)")
@@ -155,6 +158,8 @@ if __name__ == '__main__':
             config.tuned = ''
         op_name, case = config.cases[case_keys[i]]
         print(case)
+        if args.incumbents:
+            config.incumbents = [os.path.abspath(os.path.join(args.incumbents, case_keys[i], 'records.txt'))]
         env = Env(measure_option, config)
         latency = run(op_name, case_keys[i], case + [config.in_dtype, config.out_dtype], env, runner, args.check)
         cases.append([case, latency])

@@ -3,6 +3,8 @@ import ctypes
 import os
 import re
 
+import numpy as np
+
 from heron_amd import backend as B
 from heron_amd import instances
 
@@ -29,6 +31,7 @@ def header_struct(name):
     """(field name, C type, array length) of every member of ``struct name`` in the header, in declaration order."""
     text = open(os.path.join(ROOT, "include", "heron_rocm.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    macros = dict(re.findall(r"#define (HRN_\w+) (\d+)", text))
     body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (name, name), text, flags=re.S).group(1)
     out = []
     for decl in body.split(";"):
@@ -37,8 +40,9 @@ def header_struct(name):
             continue
         ctype, names = re.match(r"((?:u?int\d+_t|size_t|char|(?:const\s+)?void\s*\*))\s*(.*)", decl, flags=re.S).groups()
         for n in names.split(","):
-            m = re.match(r"\s*(\w+)(?:\[(\d+)\])?\s*$", n)
-            out.append((m.group(1), ctype.replace(" ", ""), int(m.group(2) or 0)))
+            m = re.match(r"\s*(\w+)((?:\[\w+\])*)\s*$", n)
+            dims = [int(macros.get(x, x)) for x in re.findall(r"\[(\w+)\]", m.group(2))]
+            out.append((m.group(1), ctype.replace(" ", ""), int(np.prod(dims)) if dims else 0))
     return out
 
 
@@ -49,12 +53,16 @@ C_TYPES = {"int32_t": ctypes.c_int32, "int64_t": ctypes.c_int64, "uint64_t": cty
 def test_struct_layouts_match_header():
     """Every ctypes structure has the header's members, in the header's order, with the header's types."""
     for name, cls in (("hrn_kernel_desc", B.KernelDesc), ("hrn_kernel_info", B.KernelInfo), ("hrn_problem", B.Problem),
-                      ("hrn_devinfo", B.DevInfo)):
+                      ("hrn_devinfo", B.DevInfo), ("hrn_gather", B.Gather)):
         want = [(n, C_TYPES[t] * k if k else C_TYPES[t]) for n, t, k in header_struct(name)]
         have = [(n, t) for n, t in cls._fields_]
         assert [n for n, _ in have] == [n for n, _ in want], name
         for (n, th), (_, tw) in zip(have, want):
-            assert ctypes.sizeof(th) == ctypes.sizeof(tw) and th._type_ == tw._type_, (name, n)
+            def scalar(t):
+                while hasattr(t, "_length_"):
+                    t = t._type_                                     # element type of a (nested) array
+                return t._type_
+            assert ctypes.sizeof(th) == ctypes.sizeof(tw) and scalar(th) == scalar(tw), (name, n)
     assert ctypes.sizeof(B.KernelDesc) == 18 * 4
     assert B.KernelDesc.KEYS == tuple(n for n, _ in B.KernelDesc._fields_)
 
@@ -134,3 +142,22 @@ def test_prestage_entry_points_reject_bad_arguments_without_a_gpu():
     assert L.hrn_probe_launch(0, 10, ctypes.byref(out), None) == B.HRN_E_BADPARAM
     assert L.hrn_probe_launch(256, 10, None, None) == B.HRN_E_BADPARAM
     assert L.hrn_probe_read(p, 24, 1, ctypes.byref(out), None) == B.HRN_E_BADPARAM   # not a multiple of 16 bytes
+
+
+def test_gather_rejects_bad_maps_without_a_gpu():
+    L = B.lib()
+    buf = ctypes.create_string_buffer(256)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    g = B.make_gather(2, (4, 8), [(4, 8, {0: 1}), (8, 1, {1: 1})])
+    assert (g.ndim, g.nsrc, g.dst_stride[0], g.dst_stride[1], g.dst_live[1], g.mul[0][0], g.mul[1][1], g.div[0]) == (2, 2, 8, 1, 8, 1, 1, 1)
+    assert L.hrn_gather_nd(None, p, None, p, None) == B.HRN_E_BADPARAM
+    g.dst_stride[1] = 2
+    assert L.hrn_gather_nd(ctypes.byref(g), p, None, p, None) == B.HRN_E_BADPARAM and b"stride 1" in L.hrn_last_error()
+    g = B.make_gather(2, (4, 8), [(4, 8, {0: 1}), (8, 1, {1: 1}, 0, 0)])                    # divisor 0
+    assert L.hrn_gather_nd(ctypes.byref(g), p, None, p, None) == B.HRN_E_BADPARAM and b"divisor" in L.hrn_last_error()
+    g = B.make_gather(2, (4, 8), [(4, 8, {0: 1}), (8, 1, {1: 1})], dst_live=(4, 9))         # live beyond the extent
+    assert L.hrn_gather_nd(ctypes.byref(g), p, None, p, None) == B.HRN_E_BADPARAM
+    g = B.make_gather(2, (4, 8), [(4, 8, {0: 1}), (8, 1, {1: 1})], op=B.GATHER_CENTER_SQUARE)   # no aux tensor
+    assert L.hrn_gather_nd(ctypes.byref(g), p, None, p, None) == B.HRN_E_BADPARAM
+    g = B.make_gather(2, (0, 8), [(4, 8, {0: 1}), (8, 1, {1: 1})])                          # nothing to do is not an error
+    assert L.hrn_gather_nd(ctypes.byref(g), p, None, p, None) == 0

@@ -227,3 +227,50 @@ def test_transpose_pad_kernel(hrn):
         B.transpose_pad(x.data_ptr(), x.data_ptr(), 1, 8, 8, 4, 2, st)             # padded rows fewer than rows
     with pytest.raises(B.HeronRocmError):
         B.transpose_pad(x.data_ptr(), x.data_ptr(), 1, 8, 8, 8, 3, st)             # 3-byte elements
+
+
+def test_gather_kernel_against_the_torch_formulation(hrn):
+    """The affine gather pass of the library (hrn_gather_nd): every adapter half that uses it, on device tensors, equals
+    the torch formulation of the same pre-stage on the host copy bit for bit - 16-byte pieces (channel counts that are
+    multiples of 8, aligned maps) and single elements (everything else), fp16 and bytes, the fused (x - mean)^2 included."""
+    import torch
+
+    def both(fn, name, args, dtype, *host):
+        info, _ = declare(name, args, dtype)
+        print("gather", name, args, dtype, flush=True)
+        want = fn(info, *[torch.from_numpy(np.ascontiguousarray(h)) for h in host])
+        got = fn(info, *[dev(h) for h in host])
+        torch.cuda.synchronize()
+        assert got.is_cuda and got.is_contiguous() and got.shape == want.shape
+        assert torch.equal(got.cpu(), want), (name, args)
+
+    for shape in [(4, 64, 14, 14), (3, 20, 7, 9), (1, 5, 3, 3), (2, 16, 8, 8)]:
+        In, Mean = rnd(shape, 30, "float16"), rnd(shape, 31, "float16")
+        both(hostops._act_mean, "mean", list(shape), "float16", In)
+        both(hostops._act_var, "var", list(shape), "float16", In, Mean)
+    for dtype in ("float16", "int8"):
+        adt = "float16" if dtype == "float16" else "uint8"
+        for ci in (5, 8, 16):
+            for s, p, d in [(1, 1, 1), ((2, 1, 1), (1, 1, 0), 1), (1, (0, 2, 1), (2, 2, 1))]:
+                X, F = rnd((2, 6, 9, 7, ci), 32, adt), rnd((3, 3, 2, ci, 16), 33, dtype)
+                both(hostops._act_c3d_ndhwc, "c3d_ndhwc", [2, 6, 9, 7, ci, 16, 3, 3, 2, s, p, d], dtype, X, F)
+        for ci in (6, 16):
+            for s, p, d, op in [(2, 1, 1, 0), (2, 1, 1, 1), (1, 0, 1, 0), (3, 2, 2, 1)]:
+                X, F = rnd((2, ci, 5, 6), 34, adt), rnd((4, ci, 3, 4), 35, dtype)
+                both(hostops._act_t2d_nchw, "t2d", [2, 5, 6, ci, 4, 3, 4, s, p, d, op], dtype, X, F)
+        for s, p, mult in [(1, 1, 1), (2, 1, 2)]:
+            X, F = rnd((2, 6, 9, 8), 36, adt), rnd((6 * mult, 3, 3), 37, dtype)
+            both(hostops._act_dep, "dep", [2, 9, 8, 6, 6 * mult, 3, 3, s, p, 1], dtype, X, F)
+    # argument checks
+    x = torch.zeros(64, dtype=torch.float16, device="cuda")
+    g = B.make_gather(2, (4, 8), [(4, 8, {0: 1}), (8, 1, {1: 1})])
+    B.gather_nd(g, x.data_ptr(), x.data_ptr())
+    g.dst_stride[1] = 2
+    with pytest.raises(B.HeronRocmError, match="stride 1"):
+        B.gather_nd(g, x.data_ptr(), x.data_ptr())
+    g = B.make_gather(2, (4, 8), [(4, 8, {0: 1}), (8, 1, {1: 1})], op=B.GATHER_CENTER_SQUARE)
+    with pytest.raises(B.HeronRocmError, match="aux"):
+        B.gather_nd(g, x.data_ptr(), x.data_ptr())
+    g = B.make_gather(3, (4, 8), [(4, 8, {0: 1}), (8, 1, {1: 1})])
+    with pytest.raises(B.HeronRocmError):
+        B.gather_nd(g, x.data_ptr(), x.data_ptr())

@@ -106,3 +106,77 @@ def test_depthwise(s, p, mult):
     assert tuple(A.shape) == (g['batch'], g['M'], g['K']) and tuple(Bm.shape) == (g['batch'], g['N'], g['K'])
     C = oracle.bmm_f32(A.numpy(), Bm.numpy())
     close(fin(c.info, torch.from_numpy(C)).numpy(), oracle.depthwise_conv2d_ref(X, F, s, p))
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The index maps the adapters hand to the library's gather pass (hrn_gather_nd), evaluated here by a plain loop over
+# the destination index space: with device tensors the adapters build these maps instead of calling torch, so the
+# maps must yield what the torch formulation of the same pre-stage yields.
+def emulate_gather(src, out, dst_dim, coords, dst_stride=None, dst_live=None, op=0, aux=None):
+    import itertools
+    s_flat, o_flat = src.reshape(-1).numpy(), out.reshape(-1).numpy()
+    a_flat = aux.reshape(-1).numpy() if aux is not None else None
+    nd = len(dst_dim)
+    if dst_stride is None:
+        dst_stride = [int(np.prod(dst_dim[d + 1:])) for d in range(nd)]
+    live_ext = dst_live if dst_live is not None else dst_dim
+    assert dst_stride[-1] == 1
+    for idx in itertools.product(*[range(int(e)) for e in dst_dim]):
+        doff = sum(i * st for i, st in zip(idx, dst_stride))
+        live = all(i < l for i, l in zip(idx, live_ext))
+        soff = 0
+        for entry in coords:
+            extent, stride, muls = entry[0], entry[1], entry[2]
+            add = entry[3] if len(entry) > 3 else 0
+            div = entry[4] if len(entry) > 4 else 1
+            num = add + sum(m * idx[d] for d, m in muls.items())
+            if num < 0 or num % div or num // div >= extent:
+                live = False
+            soff += (num // div) * stride
+        if not live:
+            o_flat[doff] = 0
+        elif op == 0:
+            o_flat[doff] = s_flat[soff]
+        else:
+            d = np.float16(s_flat[soff] - a_flat[soff])
+            o_flat[doff] = np.float16(d * d)
+    return out
+
+
+def both_paths(monkeypatch, fn, info, *tensors):
+    """The adapter half ``fn`` through its torch formulation and through the emulated library passes."""
+    via_torch = fn(info, *tensors)
+    with monkeypatch.context() as m:
+        m.setattr(hostops, "_native_ok", lambda t: True)
+        m.setattr(hostops, "_gather", emulate_gather)
+        m.setattr(hostops, "_channels_last", lambda x3, cp=None: hostops._pad_last(x3.permute(0, 2, 1), cp or x3.shape[1]))
+        via_maps = fn(info, *tensors)
+    assert via_maps.shape == via_torch.shape and via_maps.is_contiguous()
+    assert torch.equal(via_maps, via_torch)
+
+
+def info_of(name, args):
+    c = Ctx()
+    getOpFromName(name)(c, *args, "float16", "float16")
+    return c.info
+
+
+def test_gather_maps_equal_the_torch_formulation(monkeypatch):
+    t = lambda shape, seed: torch.from_numpy(rnd(shape, seed))
+    In = t((3, 10, 4, 6), 20)
+    both_paths(monkeypatch, hostops._act_mean, info_of("mean", [3, 10, 4, 6]), In)
+    both_paths(monkeypatch, hostops._act_var, info_of("var", [3, 10, 4, 6]), In, t((3, 10, 4, 6), 21))
+    In = t((1, 5, 3, 3), 22)                                    # N*H*W = 9: the rows of A are padded to 16
+    both_paths(monkeypatch, hostops._act_mean, info_of("mean", [1, 5, 3, 3]), In)
+    for s, p, d in [(1, 1, 1), ((2, 1, 1), (1, 1, 0), 1), (1, (0, 2, 1), (2, 2, 1))]:
+        X, F = t((2, 6, 5, 4, 5), 23), t((3, 3, 2, 5, 12), 24)
+        both_paths(monkeypatch, hostops._act_c3d_ndhwc, info_of("c3d_ndhwc", [2, 6, 5, 4, 5, 12, 3, 3, 2, s, p, d]), X, F)
+    for s, p, d, op in [(2, 1, 1, 0), (2, 1, 1, 1), (1, 0, 1, 0), (3, 2, 2, 1)]:
+        X, F = t((2, 6, 5, 6), 25), t((4, 6, 3, 4), 26)
+        both_paths(monkeypatch, hostops._act_t2d_nchw, info_of("t2d", [2, 5, 6, 6, 4, 3, 4, s, p, d, op]), X, F)
+    for s, p, mult in [(1, 1, 1), (2, 1, 2)]:
+        X, F = t((2, 6, 9, 8), 27), t((6 * mult, 3, 3), 28)
+        info = info_of("dep", [2, 9, 8, 6, 6 * mult, 3, 3, s, p, 1])
+        both_paths(monkeypatch, hostops._act_dep, info, X, F)
+        g = info['gemm_view']
+        both_paths(monkeypatch, hostops._fin_dep, info, t((g['batch'], g['M'], g['N']), 29))

@@ -420,7 +420,7 @@ def test_shipped_tuned_records_reinstantiate(rel, op, shape, dtype):
 def test_refinement_rounds_measure_one_knob_neighbours(tmp_path, capsys):
     """CGA spends the last quarter of its measuring rounds on the one-knob neighbourhood of the best measured points:
     every neighbour is a feasible point that differs from one of the incumbents in exactly one knob, or is the incumbent
-    with its wave grid transposed."""
+    with its wave grid transposed, or one of the operator's coupled moves."""
     env = make_env(tmp_path, method="CGA", trials=48)
     np.random.seed(2)
     random.seed(2)
@@ -440,8 +440,11 @@ def test_refinement_rounds_measure_one_knob_neighbours(tmp_path, capsys):
         vals = s.knob_manager.solved_knob_vals_phenotype
         assert s.valid and solver.SATScore(vals) == 0
         diffs = [[n for n in names if vals[n] != top[n]] for top in tops]
-        # one knob away from an incumbent (it may coincide with the other one), or its transposed wave grid
-        assert any(len(d) == 1 or (d and all(n.endswith(("wave_m", "wave_n", "tile_m", "tile_n")) for n in d)) for d in diffs)
+        # one knob away from an incumbent (it may coincide with the other one), its transposed wave grid, or one of the
+        # operator's coupled moves (other MFMA edge at the same block tile; other row length, stage count and swizzle)
+        coupled = (("wave_m", "wave_n", "tile_m", "tile_n"), ("mfma", "tile_m", "tile_n", "lds_swizzle"),
+                   ("block_k_bytes", "lds_stages", "lds_swizzle"))
+        assert any(len(d) == 1 or (d and any(all(n.endswith(c) for n in d) for c in coupled)) for d in diffs)
     # the share is a config key read at run time; 0 gives the plain loop, and so does any tuner but the constrained GA
     env.config.refine_share = 0
     assert t.refinement_share() == 0.0
@@ -518,11 +521,12 @@ def test_confirmation_phase_retimes_the_best_tiles_and_apply_best_prefers_it(tmp
     rows = [json.loads(line) for line in open(path)]
     confirmed = [r for r in rows if r.get("confirmed")]
     plain = [r for r in rows if not r.get("confirmed")]
-    assert 24 <= len(plain) <= 32 and 3 <= len(confirmed) <= 12
+    assert 24 <= len(plain) <= 32 and 3 <= len(confirmed) <= 24
     key = lambda r: (r["param"]["V#ST:dense,AX:None,VA:block_m"], r["param"]["V#ST:dense,AX:None,VA:block_n"],
                      r["param"]["P#ST:dense,AX:None,PA:block_k_bytes"])
     tiles = {key(r) for r in confirmed}
-    assert len({tuple(sorted(t[:2])) + t[2:] for t in tiles}) <= 3          # (a transposed wave grid transposes a non-square tile)
+    # three block tiles (a transposed wave grid transposes a non-square tile; a coupled move changes the row length)
+    assert len({tuple(sorted(t[:2])) for t in tiles}) <= 3
     # every confirmed row is a feasible point; the best tiles of the search are among them
     best_plain = max(plain, key=lambda r: r["perf"])
     assert key(best_plain) in {key(r) for r in confirmed}
@@ -542,6 +546,15 @@ def test_confirmation_phase_retimes_the_best_tiles_and_apply_best_prefers_it(tmp
     # other tuners have no such phase
     from heron_amd.tuner.random_tuner import CRandTuner
     assert CRandTuner(env.config).confirmation_tiles() == 0
+    # the best rows of an earlier search's records join the candidates of a later search's confirmation
+    env2 = make_env(tmp_path / "second", method="CGA", trials=16)
+    env2.config.confirm_tiles, env2.config.incumbents = 1, [path]
+    np.random.seed(6)
+    random.seed(6)
+    env2.tune("T1")
+    rows2 = [json.loads(line) for line in open(os.path.join(env2.config.log_dir, "records.txt"))]
+    codes2 = {r["code"] for r in rows2 if r.get("confirmed")}
+    assert best_conf["code"] in codes2
 
 
 def test_problem_travels_to_the_measurement_server_without_its_device_pointers():
@@ -568,3 +581,41 @@ def test_variable_ranking_follows_the_boosters_feature_weights():
     assert anaCostModel(Model, list('abcde')) == ['c', 'd', 'a', 'b', 'e']
     Model.bst = None
     assert sorted(anaCostModel(Model, list('abcde'))) == list('abcde')
+
+
+def test_coupled_moves_reach_the_other_row_length_and_the_other_mfma_edge():
+    """From a 256x256 tile with 64-byte rows, four stages and 16x16 MFMAs, the refinement neighbourhood contains the same
+    block tile with 128-byte rows and two stages, and the same block tile built from 32x32 MFMAs: feasible points that
+    are three knobs away, so no one-knob move finds them."""
+    from heron_amd.sample import Sample
+    cfg = Config()
+    cfg.codegen_type = 'GPU_MFMA'
+    t = Task("t", getOpFromName("gemm"), [8192, 8192, 8192, "int8", "int8"], "rocm")
+    t.config = cfg
+    t.make_stage_schedules()
+    km = Sample(t).knob_manager
+    names = km.knob_names
+    want = dict(mfma=16, wave_m=4, wave_n=2, tile_m=4, tile_n=8, block_k_bytes=64, lds_stages=4, lds_swizzle=3, persistent=0,
+                split_k=1, conv_window=0, epilogue=1, column_sums=1)
+    knobs = {}
+    for n in names:
+        short = n.split("PA:")[-1]
+        knobs[n] = want.get(short, km.get_knob_candidates(n)[0])
+    point, valid = km.validate(knobs)
+    assert valid
+    labelled = t.coupled_moves(km)
+    assert {label for label, _ in labelled} == {"mfma=32", "block_k_bytes=128", "block_k_bytes=256"}
+    moves = [m for _, m in labelled]
+
+    def short(d):
+        return {n.split("PA:")[-1]: v for n, v in d.items()}
+
+    feasible = []
+    for m in moves:
+        p, ok = Sample(t).knob_manager.validate(m)
+        if ok:
+            feasible.append(short(m))
+    assert any(m['block_k_bytes'] == 128 and m['lds_stages'] == 2 and m['mfma'] == 16 and m['tile_m'] == 4 for m in feasible)
+    assert any(m['mfma'] == 32 and m['tile_m'] == 2 and m['tile_n'] == 4 and m['block_k_bytes'] == 64 for m in feasible)
+    # every move keeps the block tile: rows per wave tile x wave grid unchanged
+    assert all(m['tile_m'] * m['mfma'] == 64 and m['tile_n'] * m['mfma'] == 128 for m in map(short, moves))
