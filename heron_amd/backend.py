@@ -66,10 +66,10 @@ class KernelDesc(ctypes.Structure):
                 ("stages", ctypes.c_int32), ("swizzle", ctypes.c_int32), ("epilogue", ctypes.c_int32),
                 ("waves_per_eu", ctypes.c_int32), ("conv_window", ctypes.c_int32), ("persistent", ctypes.c_int32),
                 ("split_k", ctypes.c_int32), ("sched", ctypes.c_int32),
-                ("load_spread", ctypes.c_int32), ("colsum", ctypes.c_int32)]
+                ("load_spread", ctypes.c_int32), ("colsum", ctypes.c_int32), ("nt_store", ctypes.c_int32)]
 
     KEYS = ("dtype", "op", "bm", "bn", "bkb", "wm", "wn", "mfma", "stages", "swizzle", "epilogue", "waves_per_eu",
-            "conv_window", "persistent", "split_k", "sched", "load_spread", "colsum")
+            "conv_window", "persistent", "split_k", "sched", "load_spread", "colsum", "nt_store")
 
     def as_tuple(self):
         return tuple(int(getattr(self, k)) for k in self.KEYS)
@@ -102,9 +102,10 @@ class Problem(ctypes.Structure):
 
 
 def make_desc(dtype, op=HRN_OP_GEMM, bm=128, bn=128, bkb=128, wm=2, wn=2, mfma=32, stages=2, swizzle=1,
-              epilogue=0, waves_per_eu=0, conv_window=0, persistent=0, split_k=0, sched=1, load_spread=2, colsum=0):
+              epilogue=0, waves_per_eu=0, conv_window=0, persistent=0, split_k=0, sched=1, load_spread=2, colsum=0, nt_store=0):
     d = KernelDesc()
     d.colsum = colsum
+    d.nt_store = nt_store
     d.conv_window, d.persistent, d.split_k, d.sched, d.load_spread = conv_window, persistent, split_k, sched, load_spread
     d.dtype, d.op, d.bm, d.bn, d.bkb, d.wm, d.wn = dtype, op, bm, bn, bkb, wm, wn
     d.mfma, d.stages, d.swizzle, d.epilogue, d.waves_per_eu = mfma, stages, swizzle, epilogue, waves_per_eu

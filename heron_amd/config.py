@@ -21,6 +21,8 @@ DEFAULTS = {
     'refine_share': 0.25,
     # constrained GA: block tiles whose best points are re-timed with long repeats when the search is over (0 = off)
     'confirm_tiles': 8,
+    # ... and rounds in which the one-knob neighbours of the best confirmed point are timed the same way
+    'polish_rounds': 1,
     # constrained GA: records files of earlier searches whose best rows the confirmation phase times again
     'incumbents': (),
     # simulated annealing
@@ -40,7 +42,7 @@ REQUIRED_KEYS = {'out_name': 'out_name', 'method': 'opt_method', 'max_trials': '
                  'build_timeout': 'build_timeout', 'in_dtype': 'in_dtype', 'out_dtype': 'out_dtype', 'cases': 'cases'}
 # optional keys; all but "temperature" are additions of this build
 OPTIONAL_KEYS = ('temperature', 'pop_num', 'iter_walks', 'parallel_num', 'measure_time_per_round', 'select_num',
-                 'history_topk', 'refine_share', 'confirm_tiles', 'incumbents')
+                 'history_topk', 'refine_share', 'confirm_tiles', 'polish_rounds', 'incumbents')
 
 
 class Config:

@@ -10,6 +10,7 @@
 #include <signal.h>
 #include <sys/stat.h>
 #include <sys/types.h>
+#include <spawn.h>
 #include <sys/wait.h>
 #include <unistd.h>
 
@@ -51,6 +52,8 @@ struct hrn_module {
     int persist_grid;   // persistent instances: workgroups that fit the device at once (multiple of 8 when >= 8)
     int epi_bytes;      // LDS bytes of the epilogue region (column sums + strips)
 };
+
+extern char** environ;
 
 namespace {
 
@@ -148,6 +151,7 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
     if (d->split_k && d->conv_window) return fail(HRN_E_BADPARAM, "split_k uses the im2col load path, not conv_window");
     if (d->colsum < 0 || d->colsum > 1 || (d->colsum && d->dtype != HRN_DT_U8S8))
         return fail(HRN_E_BADPARAM, "colsum %d (caller-supplied column sums are an option of the u8s8 instances)", d->colsum);
+    if (d->nt_store < 0 || d->nt_store > 1) return fail(HRN_E_BADPARAM, "nt_store %d (0 or 1)", d->nt_store);
     if (d->sched == 2 && (d->wm * d->wn != 8 || d->conv_window || d->persistent || d->split_k))
         return fail(HRN_E_BADPARAM, "sched 2 (two wave groups) needs 8 waves and neither conv_window, persistent nor split_k");
     Derived r;
@@ -208,9 +212,9 @@ int derive(const hrn_kernel_desc* d, Derived* o) {
 
 std::string desc_key(const hrn_kernel_desc* d, uint64_t srch) {
     char b[256];
-    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_c%d_r%d_k%d_i%d_l%d_b%d_%08x", d->dtype, d->op, d->bm, d->bn,
+    snprintf(b, sizeof b, "hrn_d%d_o%d_m%dn%dk%d_w%dx%d_t%d_s%d_z%d_e%d_p%d_c%d_r%d_k%d_i%d_l%d_b%d_n%d_%08x", d->dtype, d->op, d->bm, d->bn,
              d->bkb, d->wm, d->wn, d->mfma, d->stages, d->swizzle, d->epilogue, d->waves_per_eu, d->conv_window,
-             d->persistent, d->split_k, d->sched, d->load_spread, d->colsum, (unsigned)(srch ^ (srch >> 32)));
+             d->persistent, d->split_k, d->sched, d->load_spread, d->colsum, d->nt_store, (unsigned)(srch ^ (srch >> 32)));
     return b;
 }
 
@@ -221,20 +225,28 @@ int parse_remark(const std::string& log, const char* tag) {
 }
 
 int run_hipcc(const std::vector<std::string>& args, const std::string& log_path, double timeout_s) {
-    // everything the child needs is prepared here: between fork and exec it only makes async-signal-safe calls
-    // (the calling process may be multi-threaded, so the child must not allocate)
+    // posix_spawn, not fork: the calling process may own a multi-threaded HIP runtime, whose address space (device
+    // mappings included) a forked child would duplicate; the spawned compiler starts from a clean image in its own
+    // process group, with the log file as stdout and stderr
     std::vector<char*> argv;
     for (auto& a : args) argv.push_back(const_cast<char*>(a.c_str()));
     argv.push_back(nullptr);
     const int fd = open(log_path.c_str(), O_WRONLY | O_CREAT | O_TRUNC | O_CLOEXEC, 0644);
-    pid_t pid = fork();
-    if (pid < 0) { if (fd >= 0) close(fd); return fail(HRN_E_BUILD, "fork failed"); }
-    if (pid == 0) {
-        setpgid(0, 0);
-        if (fd >= 0) { dup2(fd, 1); dup2(fd, 2); }
-        execvp(argv[0], argv.data());
-        _exit(127);
+    posix_spawn_file_actions_t fa;
+    posix_spawnattr_t at;
+    posix_spawn_file_actions_init(&fa);
+    posix_spawnattr_init(&at);
+    if (fd >= 0) {
+        posix_spawn_file_actions_adddup2(&fa, fd, 1);
+        posix_spawn_file_actions_adddup2(&fa, fd, 2);
     }
+    posix_spawnattr_setflags(&at, POSIX_SPAWN_SETPGROUP);
+    posix_spawnattr_setpgroup(&at, 0);
+    pid_t pid = -1;
+    const int sp = posix_spawnp(&pid, argv[0], &fa, &at, argv.data(), environ);
+    posix_spawn_file_actions_destroy(&fa);
+    posix_spawnattr_destroy(&at);
+    if (sp != 0) { if (fd >= 0) close(fd); return fail(HRN_E_BUILD, "cannot start %s: %s", argv[0], strerror(sp)); }
     if (fd >= 0) close(fd);
     auto t0 = std::chrono::steady_clock::now();
     int status = 0;
@@ -298,6 +310,7 @@ int compile_desc(const hrn_kernel_desc* d, double timeout_s, std::string* out_pa
     def("HRN_SCHED", d->sched);
     def("HRN_LSPREAD", d->load_spread);
     def("HRN_COLSUM", d->colsum);
+    def("HRN_NTSTORE", d->nt_store);
     {
         std::stringstream es(extra);
         std::string tok;

@@ -90,6 +90,13 @@ constexpr bool SPLITK = (HRN_SPLITK != 0);
 #define HRN_COLSUM 0
 #endif
 constexpr bool COLSUM = (HRN_DTYPE == 1) && (HRN_COLSUM != 0);
+// the results leave with the non-temporal hint: C is written once and not read by this kernel, and a round's 8 MiB of it
+// per XCD would otherwise push the operand slabs of the next round out of the 4 MiB L2 (split-K partial sums, which the
+// reduction reads right away, keep the default policy)
+#ifndef HRN_NTSTORE
+#define HRN_NTSTORE 0
+#endif
+constexpr bool NTS = (HRN_NTSTORE != 0) && (HRN_SPLITK == 0);
 // Issue order of a k-step: 1 = the source order of the row groups is pinned (a scheduling fence after every row of
 // MFMAs), 0 = the compiler interleaves on its own, guided by group hints (one LDS read per few MFMAs), 2 = the two
 // wave groups of an 8-wave workgroup alternate between a memory phase and a matrix phase (see "SCHED 2" below).
@@ -648,6 +655,10 @@ hrn_mfma_kernel(const HrnKArgs a) {
         };
 
         char* Cb = (char*)a.C + ((int64_t)slice * a.batch + c_bz) * a.sC * OES;
+        auto put = [&](auto* ptr, auto val) __attribute__((always_inline)) {
+            if constexpr (NTS) __builtin_nontemporal_store(val, ptr);
+            else *ptr = val;
+        };
         if constexpr (EPI >= 1) {
             // LDS-staged epilogue: a wave parks one MFMA row-tile (MT rows x SW columns) of its result in a private,
             // padded LDS strip, then streams it out with 16 bytes per lane_e, whole row segments per store instruction.
@@ -698,12 +709,12 @@ hrn_mfma_kernel(const HrnKArgs a) {
                         if constexpr (PERS) {
                             // always issued, so that every wave has exactly STORES_PER_TILE stores per tile in flight
                             const uint32_t off = (m < a.M && n + EPC <= a.N) ? (uint32_t)(m * a.ldc + n) * OES : OOB;
-                            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(unsigned int __attribute__((ext_vector_type(4))), val), rsrcC, (int)off, 0, 0);
+                            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(unsigned int __attribute__((ext_vector_type(4))), val), rsrcC, (int)off, 0, NTS ? 2 : 0);
                         } else {
                             char* dst = Cb + ((int64_t)m * a.ldc + n) * OES;
                             if (m < a.M) {
-                                if (n + EPC <= a.N) *(v4i*)dst = val;
-                                else if (OES == 2 && n + 4 <= a.N) *(long*)dst = ((long)(uint32_t)val.y << 32) | (uint32_t)val.x;
+                                if (n + EPC <= a.N) put((v4i*)dst, val);
+                                else if (OES == 2 && n + 4 <= a.N) put((long*)dst, (long)(((long)(uint32_t)val.y << 32) | (uint32_t)val.x));
                             }
                         }
                     }
@@ -726,18 +737,18 @@ hrn_mfma_kernel(const HrnKArgs a) {
                                 v4h o;
 #pragma unroll
                                 for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[i][j][g * 4 + r];
-                                *(v4h*)dst = o;
+                                put((v4h*)dst, o);
                             } else if constexpr (DT == 0) {
                                 v4f o;
 #pragma unroll
                                 for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r];
-                                *(v4f*)dst = o;
+                                put((v4f*)dst, o);
                             } else {
                                 const v4i bs = colsum4(nl);
                                 v4i o;
 #pragma unroll
                                 for (int r = 0; r < 4; ++r) o[r] = acc[i][j][g * 4 + r] + 128 * bs[r];
-                                *(v4i*)dst = o;
+                                put((v4i*)dst, o);
                             }
                         }
                     }

@@ -12,8 +12,8 @@ F16, U8 = B.HRN_DT_F16, B.HRN_DT_U8S8
 GEMM, CONV = B.HRN_OP_GEMM, B.HRN_OP_CONV2D
 
 
-def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, win=0, pers=0, split=0, sched=1, spread=2, colsum=0):
-    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, win, pers, split, sched, spread, colsum)
+def D(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi=0, wpe=0, win=0, pers=0, split=0, sched=1, spread=2, colsum=0, nt=0):
+    return B.make_desc(dtype, op, bm, bn, bkb, wm, wn, mfma, stages, swz, epi, wpe, win, pers, split, sched, spread, colsum, nt)
 
 
 # (bm, bn, bkb, wm, wn, mfma, stages, swizzle): a spread of the template space used by the parity tests
@@ -62,6 +62,10 @@ def variant_descs():
     out.append(D(U8, GEMM, 128, 128, 64, 2, 4, 16, 4, 3, epi=1, sched=2))
     out.append(D(F16, GEMM, 128, 256, 64, 2, 4, 32, 3, 2, sched=2))
     out.append(D(F16, CONV, 128, 64, 128, 4, 2, 16, 2, 1, epi=1, sched=2))
+    # non-temporal result stores: direct and staged epilogues, both element types
+    out.append(D(F16, GEMM, 128, 128, 128, 2, 2, 32, 2, 1, nt=1))
+    out.append(D(F16, GEMM, 256, 256, 128, 2, 4, 16, 2, 2, epi=2, nt=1))
+    out.append(D(U8, GEMM, 128, 128, 128, 2, 2, 16, 2, 1, epi=1, colsum=1, nt=1))
     # column sums of B supplied by the caller (colsum 1): plain, staged epilogue, two-group schedule
     out.append(D(U8, GEMM, 256, 256, 128, 2, 4, 16, 2, 1, colsum=1))
     out.append(D(U8, GEMM, 64, 128, 256, 1, 2, 16, 2, 1, epi=1, colsum=1))
@@ -133,6 +137,7 @@ def persistent_descs():
         D(F16, CONV, 128, 64, 128, 2, 1, 32, 2, 1, epi=1, pers=1),
         D(U8, CONV, 128, 64, 128, 2, 2, 16, 3, 1, epi=1, pers=1),
         D(U8, GEMM, 128, 128, 64, 2, 2, 32, 4, 3, epi=1, pers=1, colsum=1),
+        D(F16, GEMM, 128, 128, 64, 2, 2, 32, 4, 3, epi=1, pers=1, nt=1),
     ]
 
 

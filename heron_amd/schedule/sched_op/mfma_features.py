@@ -11,7 +11,8 @@ costs.  Before anything has been measured the estimate itself ranks the candidat
 import math
 
 KNOBS = ('mfma', 'wave_m', 'wave_n', 'tile_m', 'tile_n', 'block_k_bytes', 'conv_window', 'persistent', 'lds_stages',
-         'lds_swizzle', 'waves_per_eu', 'epilogue', 'split_k', 'raster_group_m', 'issue_order', 'load_spread', 'column_sums')
+         'lds_swizzle', 'waves_per_eu', 'epilogue', 'split_k', 'raster_group_m', 'issue_order', 'load_spread', 'column_sums',
+         'streaming_store')
 DERIVED = ('block_m', 'block_n', 'waves', 'k_steps', 'k_tiles', 'grid_m', 'grid_n', 'lds_bytes', 'window_bytes',
            'regs_per_lane', 'loads_per_tile')
 
@@ -116,7 +117,7 @@ def coupled_moves(names, values, candidates):
     """Knob assignments a few coordinated steps away from ``values`` that no one-knob change reaches, for the search's
     refinement rounds: (a) the other MFMA edge at the same block tile (tile counts rescaled), (b) another number of
     K bytes per LDS row with every stage count (what fits is decided by the constraint system), each with every LDS
-    swizzle, since the conflict-free swizzle depends on both.  ``names``: the task's knob names; ``values``: knob name ->
+    swizzle, since the conflict-free swizzle depends on both, (c) the other issue order with every load spread.  ``names``: the task's knob names; ``values``: knob name ->
     value of the incumbent; ``candidates(name)``: that knob's value list.  Returns (label, knob dictionary) pairs; moves
     with the same label differ only in the dependent choices (stages, swizzle)."""
     by = {}
@@ -136,6 +137,15 @@ def coupled_moves(names, values, candidates):
         for swz in swizzles:
             out.append(("mfma=%d" % other, dict(values, **{by['mfma']: other, by['tile_m']: tm * mfma // other,
                                                            by['tile_n']: tn * mfma // other, by['lds_swizzle']: swz})))
+    # (c) the other issue order with every load spread: the spread only acts on the pinned order, so a point found
+    # under the compiler's order carries an arbitrary one
+    if 'issue_order' in by and 'load_spread' in by:
+        for order in candidates(by['issue_order']):
+            if order == values[by['issue_order']]:
+                continue
+            for spread in candidates(by['load_spread']):
+                out.append(("issue_order=%d,load_spread=%d" % (order, spread),
+                            dict(values, **{by['issue_order']: order, by['load_spread']: spread})))
     for bkb in candidates(by['block_k_bytes']):
         if bkb == values[by['block_k_bytes']]:
             continue

@@ -32,7 +32,7 @@ class TemplateSchedule:
         return B.make_desc(dtype, op, p['bm'], p['bn'], p['bkb'], p['wm'], p['wn'], p['mfma'], p['stages'],
                            p['swizzle'], p.get('epilogue', 0), p['waves_per_eu'],
                            p.get('conv_window', 0), p.get('persistent', 0), 1 if p.get('split_k', 1) > 1 else 0,
-                           p.get('sched', 1), p.get('load_spread', 2), p.get('colsum', 0))
+                           p.get('sched', 1), p.get('load_spread', 2), p.get('colsum', 0), p.get('nt_store', 0))
 
     def to_problem(self):
         from ... import backend as B
@@ -514,6 +514,10 @@ class rasterOp(schedOp):
         s.params['sched'] = km.get_val(sc)
         s.params['load_spread'] = km.get_val(sp)
         s.params['colsum'] = km.get_val(cs)
+        # cache policy of the result stores: 1 = non-temporal (C does not displace the operand slabs in L2); split-K
+        # partial sums are read back at once and keep the default policy in either case
+        nt = self.knob(ctx, stage_name, 'streaming_store', [0, 1], 0)
+        s.params['nt_store'] = km.get_val(nt)
         ctx.addSchedDesc("raster group_m = %s, issue order = %s\n" % (s.params['group_m'], s.params['sched']))
 
 

@@ -198,14 +198,8 @@ class Tuner:
                 consider(max(members, key=lambda m: m[0].predict)[1])
         return out
 
-    def confirm(self, env, tiles, min_repeat_ms=100.0, repeat=3):
-        """Deterministic end of a search: every confirmation candidate is timed again with repeats of at least
-        ``min_repeat_ms`` and filed as a confirmed record; ``Task.apply_best`` prefers confirmed records, so the
-        instance a run ships no longer depends on which point a short measurement happened to favour."""
-        cands = self.confirmation_candidates(env, tiles)
-        if not cands:
-            return []
-        print("= ---- Confirmation : %d candidates, repeats of >= %.0f ms ---- =" % (len(cands), min_repeat_ms))
+    def _time_long(self, env, cands, min_repeat_ms, repeat):
+        """Times ``cands`` with repeats of at least ``min_repeat_ms`` and files the valid ones as confirmed records."""
         from ..runner.measure import MeasureInput
         from ..runner.runner import perf_of
         runner = env.runner.measure_option.get('runner') if isinstance(env.runner.measure_option, dict) else None
@@ -224,7 +218,51 @@ class Tuner:
             sample.valid, sample.perf = perf_of(result)
             if sample.valid:
                 env.perf_buffer.record_confirmed(sample)
-        done = sorted((s for s in cands if s.valid), key=lambda s: -s.perf)
+        return [s for s in cands if s.valid]
+
+    def one_knob_neighbours(self, env, base, skip=()):
+        """Feasible points that differ from ``base`` in exactly one knob, codes in ``skip`` left out."""
+        out, seen = [], set(skip)
+        geno = base.knob_manager.solved_knob_vals_genotype
+        names = base.knob_manager.knob_names
+        for name in names:
+            for cand in base.knob_manager.get_knob_candidates(name):
+                if cand == geno[name]:
+                    continue
+                s = Sample(env.task)
+                point, valid = s.knob_manager.validate({n: (cand if n == name else geno[n]) for n in names})
+                code = Code(point) if valid else None
+                if valid and code not in seen:
+                    seen.add(code)
+                    s.point, s.valid, s.stmt_code, s.violation = point, True, code, 0
+                    out.append(s)
+        return out
+
+    def confirm(self, env, tiles, min_repeat_ms=100.0, repeat=3):
+        """Deterministic end of a search: every confirmation candidate is timed again with repeats of at least
+        ``min_repeat_ms`` and filed as a confirmed record; ``Task.apply_best`` prefers confirmed records, so the
+        instance a run ships no longer depends on which point a short measurement happened to favour.  Then the best
+        confirmed point is polished: all its one-knob neighbours are timed the same way, ``config.polish_rounds`` times
+        at most (default 1) and only while the best point keeps moving - the fine knobs (issue order, load spread,
+        epilogue, raster group) move a tile by less than a short measurement resolves."""
+        cands = self.confirmation_candidates(env, tiles)
+        if not cands:
+            return []
+        print("= ---- Confirmation : %d candidates, repeats of >= %.0f ms ---- =" % (len(cands), min_repeat_ms))
+        done = sorted(self._time_long(env, cands, min_repeat_ms, repeat), key=lambda s: -s.perf)
+        timed = {s.stmt_code for s in cands}
+        for _ in range(int(getattr(self.config, 'polish_rounds', 1))):
+            if not done:
+                break
+            best = done[0]
+            near = self.one_knob_neighbours(env, best, skip=timed)
+            if not near:
+                break
+            print("= ---- Polish : %d one-knob neighbours of the confirmed best ---- =" % len(near))
+            timed.update(s.stmt_code for s in near)
+            done = sorted(done + self._time_long(env, near, min_repeat_ms, repeat), key=lambda s: -s.perf)
+            if done[0] is best:
+                break
         if done:
             print("confirmed best %f (latency %.6f ms)" % (done[0].perf, 1e3 * np.exp(-done[0].perf)))
         return done

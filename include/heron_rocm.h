@@ -96,6 +96,10 @@ typedef struct hrn_kernel_desc {
     int32_t colsum;       /* u8s8 only: the kernel computes (u8 - 128) x s8 on the signed MFMA and adds 128 * sum_k B[n,k];
                              0 = it adds those column sums up itself from the B fragments in its k-loop, 1 = it takes
                              them from hrn_problem.bsum (they depend on the weights alone: hrn_colsum_s8 makes them) */
+    int32_t nt_store;     /* 1 = the results are stored with the non-temporal hint, so that C (written once, never read
+                             by the kernel) does not push the operand slabs of the next round of tiles out of L2;
+                             0 = default cache policy (a consumer that reads C right away finds more of it in L2).
+                             Split-K partial sums always take the default policy */
 } hrn_kernel_desc;
 
 /* Resource usage of a built instance, for cross-checks of the constraint set. */

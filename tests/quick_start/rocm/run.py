@@ -72,11 +72,11 @@ def host_reference(op_name):
 
 def keep_best(src, dst, n):
     """Writes the rows of a search that are worth keeping to ``dst`` (what ``-t`` and the benchmark later load through
-    Task.apply_best): every row re-timed by the confirmation phase and the ``n`` best of the others, failed
+    Task.apply_best): the ``n`` best rows re-timed by the confirmation phase and the ``n`` best of the others, failed
     measurements dropped."""
     import json
     rows = [json.loads(line) for line in open(src) if line.strip()]
-    confirmed = [r for r in rows if r.get("confirmed") and r["perf"] > 0]
+    confirmed = sorted((r for r in rows if r.get("confirmed") and r["perf"] > 0), key=lambda r: -r["perf"])[:n]
     plain = sorted((r for r in rows if not r.get("confirmed") and r["perf"] > 0), key=lambda r: -r["perf"])[:n]
     os.makedirs(os.path.dirname(os.path.abspath(dst)), exist_ok=True)
     with open(dst, "w") as out:

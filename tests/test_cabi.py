@@ -63,7 +63,7 @@ def test_struct_layouts_match_header():
                     t = t._type_                                     # element type of a (nested) array
                 return t._type_
             assert ctypes.sizeof(th) == ctypes.sizeof(tw) and scalar(th) == scalar(tw), (name, n)
-    assert ctypes.sizeof(B.KernelDesc) == 18 * 4
+    assert ctypes.sizeof(B.KernelDesc) == 19 * 4
     assert B.KernelDesc.KEYS == tuple(n for n, _ in B.KernelDesc._fields_)
 
 

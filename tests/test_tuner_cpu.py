@@ -96,7 +96,7 @@ def test_every_sampled_instance_passes_the_c_side_check(op, shape, dtype):
     t = Task("t", getOpFromName(op), shape + [dtype, dtype], "rocm")
     t.config = cfg
     t.make_stage_schedules()
-    assert len(t.knob_manager.knob_names) == 17 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
+    assert len(t.knob_manager.knob_names) == 18 and t.knob_manager.sched_tups[0] == ('start', t.knob_manager.sched_tups[0][1])
     seen = set()
     for _ in range(40):
         km = copy.deepcopy(t.knob_manager)
@@ -443,7 +443,7 @@ def test_refinement_rounds_measure_one_knob_neighbours(tmp_path, capsys):
         # one knob away from an incumbent (it may coincide with the other one), its transposed wave grid, or one of the
         # operator's coupled moves (other MFMA edge at the same block tile; other row length, stage count and swizzle)
         coupled = (("wave_m", "wave_n", "tile_m", "tile_n"), ("mfma", "tile_m", "tile_n", "lds_swizzle"),
-                   ("block_k_bytes", "lds_stages", "lds_swizzle"))
+                   ("block_k_bytes", "lds_stages", "lds_swizzle"), ("issue_order", "load_spread"))
         assert any(len(d) == 1 or (d and any(all(n.endswith(c) for n in d) for c in coupled)) for d in diffs)
     # the share is a config key read at run time; 0 gives the plain loop, and so does any tuner but the constrained GA
     env.config.refine_share = 0
@@ -511,7 +511,7 @@ def test_confirmation_phase_retimes_the_best_tiles_and_apply_best_prefers_it(tmp
     transposed wave grid and the other issue order are timed again with long repeats and filed as confirmed records;
     apply_best then ships the best CONFIRMED row even when a short measurement of another point looked better."""
     env = make_env(tmp_path, method="CGA", trials=32)
-    env.config.confirm_tiles = 3
+    env.config.confirm_tiles, env.config.polish_rounds = 3, 0
     np.random.seed(5)
     random.seed(5)
     env.tune("T1")
@@ -555,6 +555,17 @@ def test_confirmation_phase_retimes_the_best_tiles_and_apply_best_prefers_it(tmp
     rows2 = [json.loads(line) for line in open(os.path.join(env2.config.log_dir, "records.txt"))]
     codes2 = {r["code"] for r in rows2 if r.get("confirmed")}
     assert best_conf["code"] in codes2
+    # ... and (polish_rounds is 1 by default) the one-knob neighbours of the best confirmed point were timed as well:
+    # every row of the polish step differs from the point it started from in the knob that was changed and in what
+    # the constraint system derives from it, and apply_best ships the best of all confirmed rows
+    out2 = capsys.readouterr().out
+    assert "Polish :" in out2 and out2.index("Polish :") > out2.index("Confirmation :")
+    n_conf = int(out2.split("Confirmation : ")[1].split(" ")[0])
+    n_polish = int(out2.split("Polish : ")[1].split(" ")[0])
+    confirmed2 = [r for r in rows2 if r.get("confirmed")]
+    assert n_polish >= 5 and len(confirmed2) == n_conf + n_polish
+    s3, _ = env2.task.apply_best(os.path.join(env2.config.log_dir, "records.txt"))
+    assert s3.params['bm'] == max(confirmed2, key=lambda r: r["perf"])["param"]["V#ST:dense,AX:None,VA:block_m"]
 
 
 def test_problem_travels_to_the_measurement_server_without_its_device_pointers():
@@ -604,7 +615,8 @@ def test_coupled_moves_reach_the_other_row_length_and_the_other_mfma_edge():
     point, valid = km.validate(knobs)
     assert valid
     labelled = t.coupled_moves(km)
-    assert {label for label, _ in labelled} == {"mfma=32", "block_k_bytes=128", "block_k_bytes=256"}
+    assert {label for label, _ in labelled if not label.startswith("issue_order")} == {"mfma=32", "block_k_bytes=128", "block_k_bytes=256"}
+    assert len({label for label, _ in labelled if label.startswith("issue_order=")}) == 4        # the other order x 4 spreads
     moves = [m for _, m in labelled]
 
     def short(d):
