@@ -702,7 +702,10 @@ __global__ void __launch_bounds__(256) gather_nd_kernel(const hrn_gather g, cons
     const IDX t = (IDX)blockIdx.x * 256 + threadIdx.x;
     if (t >= total) return;
     constexpr int V = VEC ? 16 / ES : 1;
-    int64_t idx[HRN_GATHER_DIMS];
+    // 32-bit index arithmetic when the launch is small enough for it (IDX = uint32_t: the host has checked that every
+    // extent, numerator and coordinate fits), 64-bit otherwise; the element offsets are 64-bit in both cases
+    using CO = typename std::conditional<sizeof(IDX) == 4, int32_t, int64_t>::type;
+    CO idx[HRN_GATHER_DIMS];
     IDX rem = t;
 #pragma unroll
     for (int d = HRN_GATHER_DIMS - 1; d >= 0; --d) {
@@ -710,7 +713,7 @@ __global__ void __launch_bounds__(256) gather_nd_kernel(const hrn_gather g, cons
         if (d < g.ndim) {
             const IDX ext = (IDX)(d == g.ndim - 1 ? g.dst_dim[d] / V : g.dst_dim[d]);
             const IDX q = rem / ext;
-            idx[d] = (int64_t)(rem - q * ext) * (d == g.ndim - 1 ? V : 1);
+            idx[d] = (CO)(rem - q * ext) * (d == g.ndim - 1 ? V : 1);
             rem = q;
         }
     }
@@ -719,20 +722,21 @@ __global__ void __launch_bounds__(256) gather_nd_kernel(const hrn_gather g, cons
 #pragma unroll
     for (int d = 0; d < HRN_GATHER_DIMS; ++d)
         if (d < g.ndim) {
-            doff += idx[d] * g.dst_stride[d];
-            live = live && idx[d] < g.dst_live[d];
+            doff += (int64_t)idx[d] * g.dst_stride[d];
+            live = live && idx[d] < (CO)g.dst_live[d];
         }
     int64_t soff = 0;
 #pragma unroll
     for (int s = 0; s < HRN_GATHER_DIMS; ++s)
         if (s < g.nsrc) {
-            int64_t num = g.add[s];
+            CO num = (CO)g.add[s];
 #pragma unroll
             for (int d = 0; d < HRN_GATHER_DIMS; ++d)
-                if (d < g.ndim) num += g.mul[s][d] * idx[d];
-            const int64_t q = num / g.div[s];
-            live = live && num >= 0 && q * g.div[s] == num && q < g.src_dim[s];
-            soff += q * g.src_stride[s];
+                if (d < g.ndim) num += (CO)g.mul[s][d] * idx[d];
+            const CO dv = (CO)g.div[s];
+            const CO q = dv == 1 ? num : num / dv;
+            live = live && num >= 0 && q * dv == num && q < (CO)g.src_dim[s];
+            soff += (int64_t)q * g.src_stride[s];
         }
     if constexpr (VEC) {
         pv4i v = {0, 0, 0, 0};
@@ -922,7 +926,19 @@ int hrn_gather_nd(const hrn_gather* g, const void* src, const void* aux, void* d
     const char* sp = (const char*)src;
     const _Float16* ap = (const _Float16*)aux;
     char* dp = (char*)dst;
-    const bool small = lanes < (1LL << 31) && total < (1LL << 31);
+    // 32-bit index arithmetic in the kernel needs every extent, divisor and reachable numerator below 2^31
+    long double reach = 0;
+    for (int sidx = 0; sidx < ns; ++sidx) {
+        long double r = g->add[sidx] < 0 ? -(long double)g->add[sidx] : (long double)g->add[sidx];
+        for (int d = 0; d < nd; ++d) {
+            const long double m = g->mul[sidx][d] < 0 ? -(long double)g->mul[sidx][d] : (long double)g->mul[sidx][d];
+            r += m * (long double)(g->dst_dim[d] ? g->dst_dim[d] - 1 : 0);
+        }
+        if (r > reach) reach = r;
+        if ((long double)g->src_dim[sidx] > reach) reach = (long double)g->src_dim[sidx];
+        if ((long double)g->div[sidx] > reach) reach = (long double)g->div[sidx];
+    }
+    const bool small = lanes < (1LL << 31) && total < (1LL << 31) && reach < 2.0e9L;
 #define HRN_GATHER_LAUNCH(ES_, VEC_)                                                                                          \
     do {                                                                                                                      \
         if (small) gather_nd_kernel<ES_, VEC_, uint32_t><<<(unsigned)blocks, 256, 0, st>>>(*g, sp, ap, dp, (uint32_t)lanes);   \
