@@ -11,6 +11,28 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+# While an OperatorPlan is being recorded, every library call of this module is also appended here (callable, arguments):
+# replaying the list repeats the device work of the call without its Python and torch bookkeeping.
+_recording = None
+
+
+_keepalive = None
+
+
+def _new(maker, *args, **kwargs):
+    """A fresh tensor; while a plan is recorded it is kept alive with the plan (the recorded calls hold addresses)."""
+    t = maker(*args, **kwargs)
+    if _keepalive is not None:
+        _keepalive.append(t)
+    return t
+
+
+def _do(fn, *args):
+    if _recording is not None:
+        _recording.append((fn, args))
+    return fn(*args)
+
+
 def _chk(t, dtype):
     if not (t.is_cuda and t.is_contiguous() and t.dtype == dtype):
         raise ValueError("expected a contiguous CUDA tensor of %s, got %s %s" % (dtype, t.dtype, t.device))
@@ -24,7 +46,7 @@ def column_sums(Bm):
         n, k, batch = Bm.shape[0], Bm.shape[1] * Bm.shape[2] * Bm.shape[3], 1
     else:
         n, k, batch = Bm.shape[-2], Bm.shape[-1], (Bm.shape[0] if Bm.dim() == 3 else 1)
-    out = torch.empty((batch, n) if Bm.dim() == 3 else (n,), dtype=torch.int32, device=Bm.device)
+    out = _new(torch.empty, (batch, n) if Bm.dim() == 3 else (n,), dtype=torch.int32, device=Bm.device)
     B.colsum_s8(Bm.data_ptr(), out.data_ptr(), batch, n, k, stream=_stream())
     return out
 
@@ -43,14 +65,14 @@ def gemm(mod, A, Bm, out=None, group_m=8, split_k=0, bsum=None):
         raise ValueError("shape mismatch %s x %s" % (tuple(A.shape), tuple(Bm.shape)))
     oshape = (batch, M, N) if A.dim() == 3 else (M, N)
     if out is None:
-        out = torch.empty(oshape, dtype=torch.float16 if f16 else torch.int32, device=A.device)
+        out = _new(torch.empty, oshape, dtype=torch.float16 if f16 else torch.int32, device=A.device)
     p = B.gemm_problem(batch, M, N, K, group_m, split_k)
     if bsum is not None and mod.desc.colsum:
         _chk(bsum, torch.int32)
         if bsum.numel() != batch * N:
             raise ValueError("bsum holds %d sums, B has %d columns" % (bsum.numel(), batch * N))
         p.bsum = bsum.data_ptr()
-    mod.launch(p, A.data_ptr(), Bm.data_ptr(), out.data_ptr(), _stream())
+    _do(mod.launch, p, A.data_ptr(), Bm.data_ptr(), out.data_ptr(), _stream())
     return out
 
 
@@ -77,13 +99,13 @@ def conv2d_nhwc(mod, X, Wt, stride=1, pad=0, dil=1, out=None, group_m=8, split_k
     ho = (H - ((KH - 1) * dh + 1) + 2 * ph) // sh + 1
     wo = (W - ((KW - 1) * dw + 1) + 2 * pw) // sw + 1
     if out is None:
-        out = torch.empty((N, ho, wo, CO), dtype=torch.float16 if f16 else torch.int32, device=X.device)
+        out = _new(torch.empty, (N, ho, wo, CO), dtype=torch.float16 if f16 else torch.int32, device=X.device)
     if bsum is not None and mod.desc.colsum:
         _chk(bsum, torch.int32)
         if bsum.numel() != CO:
             raise ValueError("bsum holds %d sums, the filter has %d output channels" % (bsum.numel(), CO))
         p.bsum = bsum.data_ptr()
-    mod.launch(p, X.data_ptr(), Wt.data_ptr(), out.data_ptr(), _stream())
+    _do(mod.launch, p, X.data_ptr(), Wt.data_ptr(), out.data_ptr(), _stream())
     return out
 
 
@@ -98,8 +120,8 @@ def _pad_last(t, to):
     if c == to:
         return t.contiguous()
     if t.is_cuda and t.is_contiguous() and t.element_size() in (1, 2) and (to * t.element_size()) % 16 == 0:
-        out = torch.empty(t.shape[:-1] + (to,), dtype=t.dtype, device=t.device)
-        B.pad_rows(t.data_ptr(), out.data_ptr(), t.numel() // c, c, to, t.element_size(), _stream())
+        out = _new(torch.empty, t.shape[:-1] + (to,), dtype=t.dtype, device=t.device)
+        _do(B.pad_rows, t.data_ptr(), out.data_ptr(), t.numel() // c, c, to, t.element_size(), _stream())
         return out
     return torch.nn.functional.pad(t, (0, to - c)).contiguous()
 
@@ -112,7 +134,7 @@ def _gather(src, out, dst_dim, coords, dst_stride=None, dst_live=None, op=B.GATH
     """One pass of the library's affine gather from ``src`` into ``out`` (both contiguous device tensors; see
     backend.make_gather for ``coords``)."""
     g = B.make_gather(src.element_size(), dst_dim, coords, dst_stride, dst_live, op)
-    B.gather_nd(g, src.data_ptr(), out.data_ptr(), aux.data_ptr() if aux is not None else None, _stream())
+    _do(B.gather_nd, g, src.data_ptr(), out.data_ptr(), aux.data_ptr() if aux is not None else None, _stream())
     return out
 
 
@@ -121,8 +143,8 @@ def _channels_last(x3, cp=None):
     N, C, L = x3.shape
     cp = cp or C
     if _native_ok(x3) and N <= 65535 and L > 0:
-        out = torch.empty((N, L, cp), dtype=x3.dtype, device=x3.device)
-        B.transpose_pad(x3.data_ptr(), out.data_ptr(), N, C, L, cp, x3.element_size(), _stream())
+        out = _new(torch.empty, (N, L, cp), dtype=x3.dtype, device=x3.device)
+        _do(B.transpose_pad, x3.data_ptr(), out.data_ptr(), N, C, L, cp, x3.element_size(), _stream())
         return out
     return _pad_last(x3.permute(0, 2, 1), cp)
 
@@ -131,8 +153,8 @@ def _channels_first(y3):
     """(N, L, C) -> (N, C, L)."""
     N, L, C = y3.shape
     if _native_ok(y3) and N <= 65535 and L > 0:
-        out = torch.empty((N, C, L), dtype=y3.dtype, device=y3.device)
-        B.transpose_pad(y3.data_ptr(), out.data_ptr(), N, L, C, L, y3.element_size(), _stream())
+        out = _new(torch.empty, (N, C, L), dtype=y3.dtype, device=y3.device)
+        _do(B.transpose_pad, y3.data_ptr(), out.data_ptr(), N, L, C, L, y3.element_size(), _stream())
         return out
     return y3.permute(0, 2, 1).contiguous()
 
@@ -154,7 +176,7 @@ def _act_pad_k(info, A, *_):
 
 def _const_gemv(info, A, b):
     g = info['gemm_view']
-    Bp = torch.zeros((g['N'], g['K']), dtype=b.dtype, device=b.device)
+    Bp = _new(torch.zeros, (g['N'], g['K']), dtype=b.dtype, device=b.device)
     Bp[0, :b.shape[-1]] = b.reshape(-1)
     return Bp
 
@@ -178,7 +200,7 @@ def _channel_major(info, In, mean=None):
             d = In - mean
             In = d * d
         return _pad_last(In.permute(1, 0, 2, 3).reshape(C, N * H * W), K)
-    out = (torch.empty if K == N * H * W else torch.zeros)((C, K), dtype=In.dtype, device=In.device)
+    out = _new(torch.empty if K == N * H * W else torch.zeros, (C, K), dtype=In.dtype, device=In.device)
     return _gather(In, out, (C, N, H * W), [(N, C * H * W, {1: 1}), (C, H * W, {0: 1}), (H * W, 1, {2: 1})],
                    dst_stride=(K, H * W, 1), op=B.GATHER_CENTER_SQUARE if mean is not None else B.GATHER_COPY, aux=mean)
 
@@ -190,7 +212,7 @@ def _act_mean(info, In, *_):
 def _const_mean(info, In, *_):
     g = info['gemm_view']
     N, C, H, W = In.shape
-    Bm = torch.zeros((g['N'], g['K']), dtype=In.dtype, device=In.device)
+    Bm = _new(torch.zeros, (g['N'], g['K']), dtype=In.dtype, device=In.device)
     Bm[0, :N * H * W] = 1.0 / (N * H * W)
     return Bm
 
@@ -249,11 +271,11 @@ def _act_c3d_ndhwc(info, X, F):           # (N,D,H,W,CI)
     cip = info['conv']['CI'] // KD
     if _native_ok(X):
         # depth taps side by side on the channel axis: channel block kd of output slice z is input slice z*sd + kd*dd - pd
-        out = torch.empty((N * DO, H, W, KD * cip), dtype=X.dtype, device=X.device)
+        out = _new(torch.empty, (N * DO, H, W, KD * cip), dtype=X.dtype, device=X.device)
         return _gather(X, out, (N, DO, H * W, KD, cip),
                        [(N, D * H * W * CI, {0: 1}), (D, H * W * CI, {1: sd, 3: dd}, -pd), (H * W, CI, {2: 1}), (CI, 1, {4: 1})],
                        dst_live=(N, DO, H * W, KD, CI))
-    Xp = torch.zeros((N, D + 2 * pd, H, W, cip), dtype=X.dtype, device=X.device)
+    Xp = _new(torch.zeros, (N, D + 2 * pd, H, W, cip), dtype=X.dtype, device=X.device)
     Xp[:, pd:pd + D, :, :, :CI] = X
     # depth taps side by side on the channel axis: channel block kd of output slice z is input slice z*sd + kd*dd
     cols = torch.stack([Xp[:, kd * dd: kd * dd + (DO - 1) * sd + 1: sd] for kd in range(KD)], dim=4)
@@ -287,11 +309,11 @@ def _act_t2d_nchw(info, X, F):            # (N,CI,H,W): zero-expanded by the str
         # channels last (and padded) first, then one pass that writes every pixel of the expanded image: input pixel
         # ((y - top) / s, (x - left) / s) where both divide, zero elsewhere
         Xc = _channels_last(X.reshape(N, CI, H * W), c['CI'])
-        Xe = torch.empty((N, c['H'], c['W'], c['CI']), dtype=X.dtype, device=X.device)
+        Xe = _new(torch.empty, (N, c['H'], c['W'], c['CI']), dtype=X.dtype, device=X.device)
         return _gather(Xc, Xe, (N, c['H'], c['W'], c['CI']),
                        [(N, H * W * c['CI'], {0: 1}), (H, W * c['CI'], {1: 1}, -top, s), (W, c['CI'], {2: 1}, -left, s),
                         (c['CI'], 1, {3: 1})])
-    Xe = torch.zeros((N, c['H'], c['W'], c['CI']), dtype=X.dtype, device=X.device)
+    Xe = _new(torch.zeros, (N, c['H'], c['W'], c['CI']), dtype=X.dtype, device=X.device)
     if s > 1:
         # channels last (and padded) first, so that the strided scatter moves whole pixels (stride 2: 137 -> 70 us end
         # to end on 16x56x56x64); with stride 1 the permuted assignment is one pass and an extra launch only costs
@@ -307,13 +329,13 @@ def _act_dep(info, X, F):                 # (N,C,H,W): the 3x3 windows as 4x4 = 
     N, C, H, W = X.shape
     s, p, HO, WO = d['stride'], d['pad'], d['HO'], d['WO']
     if _native_ok(X):
-        A = torch.empty((C, N * HO * WO, 16), dtype=X.dtype, device=X.device)
+        A = _new(torch.empty, (C, N * HO * WO, 16), dtype=X.dtype, device=X.device)
         return _gather(X, A, (C, N, HO, WO, 4, 4),
                        [(N, C * H * W, {1: 1}), (C, H * W, {0: 1}), (H, W, {2: s, 4: 1}, -p), (W, 1, {3: s, 5: 1}, -p)],
                        dst_live=(C, N, HO, WO, 3, 3))
-    Xp = torch.zeros((N, C, H + 2 * p + 1, W + 2 * p + 1), dtype=X.dtype, device=X.device)
+    Xp = _new(torch.zeros, (N, C, H + 2 * p + 1, W + 2 * p + 1), dtype=X.dtype, device=X.device)
     Xp[:, :, p:p + H, p:p + W] = X
-    A = torch.zeros((C, N, HO, WO, 4, 4), dtype=X.dtype, device=X.device)
+    A = _new(torch.zeros, (C, N, HO, WO, 4, 4), dtype=X.dtype, device=X.device)
     for r in range(3):
         for q in range(3):
             A[:, :, :, :, r, q] = Xp[:, :, r: r + (HO - 1) * s + 1: s, q: q + (WO - 1) * s + 1: s].permute(1, 0, 2, 3)
@@ -323,7 +345,7 @@ def _act_dep(info, X, F):                 # (N,C,H,W): the 3x3 windows as 4x4 = 
 def _const_dep(info, X, F):               # (K,3,3)
     d = info['dep']
     C, mult, NP = X.shape[1], d['mult'], d['NP']
-    Bm = torch.zeros((C, NP, 4, 4), dtype=F.dtype, device=F.device)
+    Bm = _new(torch.zeros, (C, NP, 4, 4), dtype=F.dtype, device=F.device)
     Bm[:, :mult, :3, :3] = F.reshape(C, mult, 3, 3)
     return Bm.reshape(C, NP, 16)
 
@@ -332,7 +354,7 @@ def _fin_dep(info, Cm):                   # (C, N*HO*WO, NP) -> (N, C, NP, HO, W
     d = info['dep']
     C, N, HW, NP = d['C'], d['N'], d['HO'] * d['WO'], d['NP']
     if _native_ok(Cm):
-        out = torch.empty((N, C, NP, d['HO'], d['WO']), dtype=Cm.dtype, device=Cm.device)
+        out = _new(torch.empty, (N, C, NP, d['HO'], d['WO']), dtype=Cm.dtype, device=Cm.device)
         return _gather(Cm, out, (N, C, NP, HW), [(C, N * HW * NP, {1: 1}), (N, HW * NP, {0: 1}), (HW, NP, {3: 1}), (NP, 1, {2: 1})])
     return Cm.reshape(d['C'], d['N'], d['HO'], d['WO'], d['NP']).permute(1, 0, 4, 2, 3).contiguous()
 
@@ -395,19 +417,72 @@ def prepare_constant(info, inputs):
     return ADAPTERS[info.get('adapter', 'identity')][1](info, *inputs)
 
 
-def run_operator(mod, info, inputs, group_m=8, split_k=0, constant=None):
+def run_operator(mod, info, inputs, group_m=8, split_k=0, constant=None, bsum=None):
     """Runs one operator of the registry on device tensors given in the reference's own layouts.
 
     ``info`` is the dictionary the operator definition handed to ``ctx.set_info``; ``mod`` an instance of the
     template that matches its kind and operator; ``constant`` a B operand from ``prepare_constant`` (made here when
-    absent)."""
+    absent); ``bsum`` its column sums (``column_sums``) for a ``colsum`` instance."""
     act, const, fin = ADAPTERS[info.get('adapter', 'identity')]
     A = act(info, *inputs)
     Bm = const(info, *inputs) if constant is None else constant
     if info['operator'] == 'conv2d_nhwc':
         c = info['conv']
         C = conv2d_nhwc(mod, A, Bm, (c['stride'], c['stride_w']), (c['pad'], c['pad_w']), (c['dil'], c['dil_w']),
-                        group_m=group_m, split_k=split_k)
+                        group_m=group_m, split_k=split_k, bsum=bsum)
     else:
-        C = gemm(mod, A, Bm, group_m=group_m, split_k=split_k)
+        C = gemm(mod, A, Bm, group_m=group_m, split_k=split_k, bsum=bsum)
     return fin(info, C)
+
+
+class OperatorPlan:
+    """One operator on fixed device tensors, recorded once and replayed: ``run()`` repeats the library passes and the
+    kernel launch of ``run_operator`` (same order, same stream, same buffers) without allocating, without building
+    index maps and without any torch call, and returns the same result tensor every time.  What a caller with
+    preallocated buffers pays per call.  The inputs are bound by address: new data goes into the same tensors.
+
+    A recording is only valid if every byte the operator moves is moved by a recorded call.  ``validate`` checks that:
+    the activation is changed in place, the operator is run eagerly and by replay, and both results must agree."""
+
+    def __init__(self, mod, info, inputs, group_m=8, split_k=0, constant=None, validate=True):
+        global _recording, _keepalive
+        if _recording is not None:
+            raise RuntimeError("an operator plan is already being recorded")
+        self.inputs = list(inputs)
+        self.constant = prepare_constant(info, inputs) if constant is None else constant
+        self.bsum = column_sums(self.constant) if mod.desc.colsum else None
+        self._keep = (mod, info)
+        stream = _stream()
+        _recording, _keepalive = steps, buffers = [], []
+        try:
+            self.out = run_operator(mod, info, self.inputs, group_m, split_k, self.constant, self.bsum)
+        finally:
+            _recording = _keepalive = None
+        self.steps, self.buffers = steps, buffers
+        self.stream = stream
+        if any(a[-1] != stream for _, a in steps):
+            raise RuntimeError("the recorded passes ran on more than one stream")
+        if validate:
+            x = self.inputs[0]
+            saved = x.clone()
+            if x.dtype == torch.float16:
+                x.mul_(-0.5)
+            else:
+                x.copy_(255 - x if x.dtype == torch.uint8 else -(x.clamp(min=-127)))
+            want = run_operator(mod, info, self.inputs, group_m, split_k, self.constant, self.bsum).clone()
+            self.out.zero_()
+            got = self.run()
+            ok = torch.equal(got, want)
+            x.copy_(saved)
+            self.run()
+            if not ok:
+                raise RuntimeError("operator plan: the replay does not reproduce the operator (a pre-stage of adapter "
+                                   "%r moves data outside the recorded passes)" % info.get('adapter', 'identity'))
+
+    def run(self):
+        if _stream() != self.stream:
+            raise RuntimeError("an operator plan replays on the stream it was recorded on")
+        for fn, args in self.steps:
+            fn(*args)
+        return self.out
+

@@ -274,3 +274,37 @@ def test_gather_kernel_against_the_torch_formulation(hrn):
     g = B.make_gather(3, (4, 8), [(4, 8, {0: 1}), (8, 1, {1: 1})])
     with pytest.raises(B.HeronRocmError):
         B.gather_nd(g, x.data_ptr(), x.data_ptr())
+
+
+def test_operator_plans_replay_what_run_operator_does(hrn):
+    """hostops.OperatorPlan: recorded once, every replay leaves in the plan's result tensor exactly what an eager
+    run_operator computes from the inputs' current contents - also after the inputs were overwritten in place (the
+    plan's own validation does that once; here it is done again with fresh data) - for every kind of adapter."""
+    import torch
+    cases = [
+        ("gemv", [100, 72], "float16", [(100, 72), (1, 72)]),
+        ("scan", [33, 40, 100], "float16", [(33, 100)]),
+        ("mean", [3, 20, 7, 9], "float16", [(3, 20, 7, 9)]),
+        ("var", [3, 20, 7, 9], "float16", [(3, 20, 7, 9), (3, 20, 7, 9)]),
+        ("c1d", [3, 57, 12, 20, 5, 2, 2, 1], "float16", [(3, 12, 57), (20, 12, 5)]),
+        ("c2d_nchw", [2, 20, 20, 3, 16, 7, 7, 2, 3, 1], "float16", [(2, 3, 20, 20), (16, 3, 7, 7)]),
+        ("c2d", [2, 20, 20, 3, 16, 7, 7, 2, 3, 1], "float16", [(2, 20, 20, 3), (16, 7, 7, 3)]),
+        ("c3d_ndhwc", [2, 6, 9, 7, 5, 12, 3, 3, 2, 1, 1, 1], "float16", [(2, 6, 9, 7, 5), (3, 3, 2, 5, 12)]),
+        ("c3d", [2, 6, 9, 7, 8, 16, 3, 3, 2, 1, 1, 1], "int8", [(2, 8, 6, 9, 7), (16, 8, 3, 3, 2)]),
+        ("t2d", [2, 5, 6, 6, 4, 3, 4, 2, 1, 1, 1], "float16", [(2, 6, 5, 6), (4, 6, 3, 4)]),
+        ("dep", [2, 9, 8, 6, 12, 3, 3, 2, 1, 1], "float16", [(2, 6, 9, 8), (12, 3, 3)]),
+        ("gemm", [70, 144, 48], "int8", [(70, 144), (48, 144)]),
+    ]
+    for name, args, dtype, shapes in cases:
+        info, _ = declare(name, args, dtype)
+        adt = "float16" if dtype == "float16" else "uint8"
+        inputs = [dev(rnd(sh, 40 + i, adt if i == 0 else dtype)) for i, sh in enumerate(shapes)]
+        mod = module(info)
+        print("plan", name, args, dtype, flush=True)
+        plan = hostops.OperatorPlan(mod, info, inputs)
+        assert plan.steps and torch.equal(plan.run(), hostops.run_operator(mod, info, inputs, constant=plan.constant))
+        inputs[0].copy_(dev(rnd(shapes[0], 77, adt)))
+        want = hostops.run_operator(mod, info, inputs, constant=plan.constant)
+        got = plan.run()
+        torch.cuda.synchronize()
+        assert got is plan.out and torch.equal(got, want), name
