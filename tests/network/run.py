@@ -19,7 +19,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests", "quick_start", "rocm"))
 
 import heron_amd.runner as HeronRunner                                # noqa: E402
 from heron_amd.environment import Env                                 # noqa: E402
-from run import makeConfig, run                                       # noqa: E402  (tests/quick_start/rocm/run.py)
+from run import keep_best, makeConfig, run                            # noqa: E402  (tests/quick_start/rocm/run.py)
 
 
 def main():
@@ -35,6 +35,12 @@ def main():
     parser.add_argument("-o", "--out", default="", help="write the per-layer table as JSON")
     parser.add_argument("-v", "--verbose", action="store_true")
     parser.add_argument("--check", action="store_true", help="verify every measured kernel against a host reference")
+    parser.add_argument("--incumbents", default="", metavar="DIR",
+                        help="DIR/<case>/records.txt of earlier searches: their best rows are timed again in the "
+                             "confirmation phase of every layer's search")
+    parser.add_argument("--keep-best", default="", metavar="DIR",
+                        help="after tuning a layer, write its confirmed rows and its 32 best other rows to "
+                             "DIR/<case>/records.txt (the form of the files under tuned/)")
     args = parser.parse_args()
 
     config = makeConfig(args)
@@ -54,8 +60,13 @@ def main():
             if os.path.exists(rec):
                 config.tuned = rec
         print(keys[i], op_name, case, flush=True)
+        inc = os.path.join(args.incumbents, keys[i], "records.txt") if args.incumbents else ""
+        config.incumbents = [os.path.abspath(inc)] if inc and os.path.exists(inc) else []
         env = Env(option, config)
+        tuned_here = not config.tuned
         latency = run(op_name, keys[i], case + [config.in_dtype, config.out_dtype], env, runner, args.check)
+        if args.keep_best and tuned_here:
+            keep_best(os.path.join(config.log_dir, "records.txt"), os.path.join(args.keep_best, keys[i], "records.txt"), 32)
         rows.append(dict(case=keys[i], op=op_name, shape=case, times=times, latency_ms=latency))
     plain = weighted = 0.0
     for r in rows:
